@@ -1,0 +1,22 @@
+"""MI355X-native multi-delta linear layer (the hot path of DeltaZip-style serving).
+
+    y = x @ W_base^T + x @ dequant(delta[id(x)])^T
+
+Python keeps the reference's operator and layer API; all arithmetic runs in hand-written HIP
+kernels for gfx950 behind the C ABI declared in include/dz_amd.h.  There is no CPU fallback.
+"""
+from .config import DeltaConfig
+from .layers import (BaseLayerWithDelta, ColumnParallelLinearWithDelta, DeltaMapping,
+                     MergedColumnParallelLinearWithDelta, MergedQKVParallelLinearWithDelta,
+                     RowParallelLinearWithDelta, convert_mapping, from_layer)
+from .ops import (add_delta, add_delta_slice, apply_delta, dequant, merge, multi_delta_linear,
+                  native_sizes, repack_gptq_to_native, segment, stacked_shapes)
+from .quant_linear import QuantLinear
+
+__all__ = [
+    "DeltaConfig", "BaseLayerWithDelta", "ColumnParallelLinearWithDelta", "DeltaMapping",
+    "MergedColumnParallelLinearWithDelta", "MergedQKVParallelLinearWithDelta",
+    "RowParallelLinearWithDelta", "convert_mapping", "from_layer", "add_delta", "add_delta_slice",
+    "apply_delta", "dequant", "merge", "multi_delta_linear", "native_sizes",
+    "repack_gptq_to_native", "segment", "stacked_shapes", "QuantLinear",
+]

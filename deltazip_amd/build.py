@@ -1,0 +1,44 @@
+"""Builds libdz_amd.so (HIP kernels + C ABI) in-tree for gfx950 with hipcc.
+
+Run as `python -m deltazip_amd.build`.  The library is written next to this file so that it
+travels with the source tree; nothing is installed into site-packages.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libdz_amd.so")
+
+SOURCES = ["dz_repack.cpp", "dz_kernels.hip", "dz_mdl32.hip", "dz_gemm.hip"]
+
+# packed fp32 VALU instructions are switched off for every device compilation in this project
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def build_library(verbose: bool = False, extra_flags=()) -> str:
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-x", "hip", *srcs, "-o", LIB]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc's host pass reports that it does not know the packed-fp32 feature; that is expected
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

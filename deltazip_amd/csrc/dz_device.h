@@ -1,0 +1,118 @@
+// Device helpers shared by the kernels of the multi-delta linear layer: vector types, the
+// 2/4-bit code unpackers, the launch parameter block and the delta fragment loader.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "dz_layout.h"
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 h16_t __attribute__((ext_vector_type(16)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
+
+// Phase timestamps for kernel tuning; compiled out unless DZ_TIMING is defined.
+#ifdef DZ_TIMING
+static __device__ unsigned long long* g_dz_ts;
+#define DZ_TS(i) do { if (lane == 0) { g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + (i)] = clock64(); if ((i) == 0) g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + 14] = wall_clock64(); if ((i) == 9) g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + 15] = wall_clock64(); } } while (0)
+#else
+#define DZ_TS(i) do { } while (0)
+#endif
+
+// ---------------------------------------------------------------------------------------------
+// code unpacking: packed 2/4-bit codes -> fp16 (q - zero), two values per instruction.
+// OR-ing a code into the mantissa of 1024.0 (0x6400) gives 1024 + q * 2^shift exactly; one packed
+// fma maps that to q - zero.
+// ---------------------------------------------------------------------------------------------
+union H2U { uint32_t u; h2_t h; };
+union H8U { uint32_t u[4]; h8_t h; u4_t v; };
+
+__device__ __forceinline__ uint32_t pkfma(uint32_t v, float mul, float add) {
+  H2U a, r;
+  a.u = v;
+  h2_t m = {(_Float16)mul, (_Float16)mul};
+  h2_t c = {(_Float16)add, (_Float16)add};
+  r.h = __builtin_elementwise_fma(a.h, m, c);
+  return r.u;
+}
+
+// 2-bit: one word holds both fragments (s = 0, 1) of a step.
+__device__ __forceinline__ void unpack2(uint32_t w, h8_t& a0, h8_t& a1) {
+  const uint32_t MAGIC = 0x64006400u;
+  const uint32_t w2 = w >> 10;
+  H8U r0, r1;
+  r0.u[0] = pkfma((w & 0x00030003u) | MAGIC, 1.0f, -1026.0f);
+  r0.u[1] = pkfma((w & 0x000C000Cu) | MAGIC, 0.25f, -258.0f);
+  r0.u[2] = pkfma((w & 0x00300030u) | MAGIC, 0.0625f, -66.0f);
+  r0.u[3] = pkfma((w & 0x00C000C0u) | MAGIC, 0.015625f, -18.0f);
+  r1.u[0] = pkfma((w & 0x03000300u) | MAGIC, 0.00390625f, -6.0f);
+  r1.u[1] = pkfma((w2 & 0x00030003u) | MAGIC, 1.0f, -1026.0f);
+  r1.u[2] = pkfma((w2 & 0x000C000Cu) | MAGIC, 0.25f, -258.0f);
+  r1.u[3] = pkfma((w2 & 0x00300030u) | MAGIC, 0.0625f, -66.0f);
+  a0 = r0.h;
+  a1 = r1.h;
+}
+
+// 4-bit: one word holds one fragment.
+__device__ __forceinline__ h8_t unpack4(uint32_t w) {
+  const uint32_t MAGIC = 0x64006400u;
+  const uint32_t w2 = w >> 8;
+  H8U r;
+  r.u[0] = pkfma((w & 0x000F000Fu) | MAGIC, 1.0f, -1032.0f);
+  r.u[1] = pkfma((w & 0x00F000F0u) | MAGIC, 0.0625f, -72.0f);
+  r.u[2] = pkfma((w2 & 0x000F000Fu) | MAGIC, 1.0f, -1032.0f);
+  r.u[3] = pkfma((w2 & 0x00F000F0u) | MAGIC, 0.0625f, -72.0f);
+  return r.h;
+}
+
+
+struct MdlParams {
+  const _Float16* x;
+  const _Float16* wb;
+  const u4_t* codes;
+  const u4_t* meta;
+  const _Float16* scales;
+  const long long* idx;
+  _Float16* y;
+  float* partials;
+  unsigned* counters;
+  unsigned* status;
+  long long codes_slot_u4, meta_slot_u4, scales_slot;
+  int T, K, N, S, G, gs;
+  int accumulate, ldy, nsplit, cb;
+  int NP, NKB, NPG;
+};
+
+constexpr int XS = DZ_KBLOCK + 8;  // LDS row stride of the staged activations, in halves
+
+template <int BITS>
+struct Frag {
+  u4_t meta;
+  u4_t code[BITS == 2 ? 1 : 2];
+};
+
+template <int BITS>
+__device__ __forceinline__ Frag<BITS> load_frag(const MdlParams& P, int d, int np, int kb,
+                                                int lane) {
+  // wavefront-uniform tile base + 16 bytes per lane
+  Frag<BITS> f;
+  const size_t tile = (size_t)np * P.NKB + kb;
+  const unsigned lo = (unsigned)lane * 16u;
+  const char* mb = (const char*)(P.meta + (size_t)d * P.meta_slot_u4 + tile * 64);
+  f.meta = __builtin_nontemporal_load((const u4_t*)(mb + lo));
+  if (BITS == 2) {
+    const char* cb = (const char*)(P.codes + (size_t)d * P.codes_slot_u4 + tile * 64);
+    f.code[0] = __builtin_nontemporal_load((const u4_t*)(cb + lo));
+  } else {
+    const char* cb = (const char*)(P.codes + (size_t)d * P.codes_slot_u4 + tile * 128);
+    f.code[0] = __builtin_nontemporal_load((const u4_t*)(cb + lo));
+    f.code[BITS == 2 ? 0 : 1] = __builtin_nontemporal_load((const u4_t*)(cb + lo + 1024));
+  }
+  return f;
+}
+
+// Launch of the T <= 32 kernel (dz_mdl32.hip).
+int dz_launch_mdl32(const MdlParams& P, int bits, bool pre, hipStream_t st, int ksplit_override);

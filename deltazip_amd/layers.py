@@ -1,0 +1,203 @@
+"""Delta layers: the state holders that wrap a base linear layer and apply per-token deltas.
+
+Mirrors the layer protocol of serving/vllm/delta/layers_marlin.py (eth-easl/deltazip):
+`BaseLayerWithDelta.{create_delta_weights, reset_delta, set_delta, set_mapping}` (:61-95), the
+stacked tensors each linear variant allocates (:311-333, 407-429, 510-534), `apply_weights` ->
+`apply_delta` (:362-373, 461-472, 559-571), `forward` returning (output, output_bias) (:251-260,
+573-597) and the `from_layer` factory (:736-750).
+
+The reference has one class per tensor-parallel linear type of its vLLM fork.  On a single GPU all
+of them compute the same thing, so the classes below share one implementation and differ only in
+what `can_replace_layer` accepts.  A base layer is any module with a fp16 `weight` of shape
+[out_features, in_features] (torch.nn.Linear fits); optional attributes `bias`, `skip_bias_add`
+and `output_sizes` are honoured as the reference honours them.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from .config import DeltaConfig
+
+ASYNC_COPY = True
+
+
+@dataclass
+class DeltaMapping:
+    """serving/vllm/delta/layers_marlin.py:46-58."""
+    # Per every token in input_ids:
+    index_mapping: Tuple[int, ...]
+    # Per sampled token:
+    prompt_mapping: Tuple[int, ...]
+
+    def __post_init__(self):
+        self.index_mapping = tuple(self.index_mapping)
+        self.prompt_mapping = tuple(self.prompt_mapping)
+
+    def __str__(self):
+        return f"index_mapping: {self.index_mapping}, prompt_mapping: {self.prompt_mapping}"
+
+
+class BaseLayerWithDelta(nn.Module):
+    def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
+        """Initializes delta matrices."""
+        ...
+
+    def reset_delta(self, index: int):
+        """Resets the delta weights at index back to 0."""
+        ...
+
+    def set_delta(self, index: int, bitwidth: int, qweight, qzeros, scales, g_idx, meta):
+        """Overwrites delta tensors at index."""
+        ...
+
+    def set_mapping(self, base_indices, sampler_indices, sampler_indices_padded, embeddings_indices,
+                    indices_len: List[int]):
+        """Sets the mapping indices."""
+        ...
+
+
+class LinearWithDelta(BaseLayerWithDelta):
+    """Shared implementation of the four linear variants."""
+
+    def __init__(self, base_layer: nn.Module) -> None:
+        super().__init__()
+        self.base_layer = base_layer
+        self.indices: Optional[torch.Tensor] = None
+        self.indices_len: Optional[List[int]] = None
+
+    # -- state ---------------------------------------------------------------------------------
+    def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
+        w = self.base_layer.weight
+        if w.dtype != torch.float16 or w.dim() != 2:
+            raise ValueError("base layer weight must be float16 [out_features, in_features]")
+        N, K = w.shape
+        self.bits = delta_config.max_bitwidth
+        self.pack_factor = delta_config.pack_factor
+        self.group_size = delta_config.group_size
+        qs, ms, ss = ops.stacked_shapes(K, N, self.bits, self.group_size)
+        self.bitwidth = [0] * max_deltas
+        self.qweight_stacked = torch.zeros((max_deltas,) + qs, dtype=torch.int32, device=w.device)
+        self.meta_stacked = torch.zeros((max_deltas,) + ms, dtype=torch.int16, device=w.device)
+        self.scales_stacked = torch.zeros((max_deltas,) + ss, dtype=torch.float16, device=w.device)
+
+    def reset_delta(self, index: int):
+        # all-zero scales make the slot contribute exactly 0 whatever the packed words hold
+        self.bitwidth[index] = 0
+        self.qweight_stacked[index] = 0
+        self.scales_stacked[index] = 0
+        self.meta_stacked[index] = 0x4444  # valid positions (0, 1) in every group
+
+    def set_delta(self, index: int, bitwidth: int, qweight: torch.Tensor, qzeros, scales: torch.Tensor,
+                  g_idx, meta: Optional[torch.Tensor]):
+        """With `meta` given, (qweight, scales, meta) are in the native layout (as
+        ops.repack_gptq_to_native returns them) and are copied into slot `index`, asynchronously
+        when they sit in pinned host memory.  With meta=None the GPTQ-style (qweight, qzeros, scales,
+        g_idx) are converted on the host first."""
+        if bitwidth != self.bits:
+            raise ValueError(f"layer was created for {self.bits}-bit deltas, got {bitwidth}")
+        if meta is None:
+            qweight, meta, scales = ops.repack_gptq_to_native(qweight, qzeros, scales, g_idx, bitwidth)
+        self.reset_delta(index)
+        self.bitwidth[index] = bitwidth
+        self.qweight_stacked[index].copy_(qweight.view(self.qweight_stacked[index].shape), non_blocking=ASYNC_COPY)
+        self.scales_stacked[index].copy_(scales.view(self.scales_stacked[index].shape), non_blocking=ASYNC_COPY)
+        self.meta_stacked[index].copy_(meta.view(self.meta_stacked[index].shape), non_blocking=ASYNC_COPY)
+
+    def set_mapping(self, base_indices: torch.Tensor, sampler_indices=None, sampler_indices_padded=None,
+                    embeddings_indices=None, indices_len: Optional[List[int]] = None):
+        # a view of the manager's buffer, re-read on the device at every call
+        self.indices = base_indices
+        self.indices_len = indices_len if indices_len is not None else [base_indices.numel()]
+
+    # -- compute -------------------------------------------------------------------------------
+    def apply_weights(self, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.apply_delta(x, self.qweight_stacked, self.scales_stacked, self.meta_stacked,
+                               self.indices[: self.indices_len[0]], self.base_layer.weight)
+
+    def forward(self, input_):
+        skip_bias_add = getattr(self.base_layer, "skip_bias_add", False)
+        base_bias = getattr(self.base_layer, "bias", None)
+        bias = base_bias if not skip_bias_add else None
+        output = self.apply_weights(input_, bias)
+        if bias is not None:
+            output = output + bias
+        output_bias = base_bias if skip_bias_add else None
+        return output, output_bias
+
+    @property
+    def weight(self):
+        return self.base_layer.weight
+
+    @property
+    def linear_weights(self):
+        return {"weight": self.base_layer.weight}
+
+    @classmethod
+    def can_replace_layer(cls, source_layer: nn.Module, delta_config: DeltaConfig, packed_modules_list: List,
+                          model_config=None) -> bool:
+        w = getattr(source_layer, "weight", None)
+        return isinstance(w, torch.Tensor) and w.dim() == 2 and len(packed_modules_list) == cls._n_packed
+
+
+class ColumnParallelLinearWithDelta(LinearWithDelta):
+    """layers_marlin.py:174-278."""
+    _n_packed = 1
+
+
+class MergedColumnParallelLinearWithDelta(LinearWithDelta):
+    """gate_proj + up_proj fused along the output dimension (layers_marlin.py:281-388)."""
+    _n_packed = 2
+
+    def create_delta_weights(self, max_deltas, delta_config, model_config=None) -> None:
+        sizes = getattr(self.base_layer, "output_sizes", None)
+        if sizes is not None and not (len(sizes) == 2 and sizes[0] == sizes[1]):
+            raise ValueError("DeltaColumnParallelLinear2Slice requires 2 slices with the same size.")
+        super().create_delta_weights(max_deltas, delta_config, model_config)
+
+
+class MergedQKVParallelLinearWithDelta(LinearWithDelta):
+    """q, k and v projections fused along the output dimension (layers_marlin.py:391-487)."""
+    _n_packed = 3
+
+
+class RowParallelLinearWithDelta(LinearWithDelta):
+    """o_proj / down_proj (layers_marlin.py:490-611)."""
+    _n_packed = 0
+
+    def apply_weights(self, x: torch.Tensor, bias=None) -> torch.Tensor:
+        if getattr(self.base_layer, "bias", None) is not None:
+            raise ValueError("RowParallelLinearWithDelta does not support bias yet.")
+        return super().apply_weights(x, None)
+
+
+_all_delta_classes = (ColumnParallelLinearWithDelta, MergedColumnParallelLinearWithDelta,
+                      MergedQKVParallelLinearWithDelta, RowParallelLinearWithDelta)
+
+
+def from_layer(layer: nn.Module, max_deltas: int, delta_config: DeltaConfig, packed_modules_list: List,
+               model_config=None) -> nn.Module:
+    """layers_marlin.py:736-750: wrap `layer` in the first delta class that accepts it."""
+    for delta_cls in _all_delta_classes:
+        if delta_cls.can_replace_layer(layer, delta_config, packed_modules_list, model_config):
+            ret = delta_cls(layer)
+            ret.create_delta_weights(max_deltas, delta_config, model_config)
+            return ret
+    return layer
+
+
+def convert_mapping(index_mapping, delta_index_to_id: List[Optional[int]], out: Optional[torch.Tensor] = None,
+                    device=None) -> torch.Tensor:
+    """Per-token delta id (0 or None = base) -> slot index (-1 = base), the part of
+    serving/vllm/delta/models.py:69-145 that feeds `set_mapping`.  Writes into `out[:T]` when given
+    (the manager's persistent buffer) and returns the [T] view."""
+    slots = [(-1 if (i is None or i <= 0) else delta_index_to_id.index(i)) for i in index_mapping]
+    t = torch.tensor(slots, dtype=torch.int64)
+    if out is not None:
+        out[: len(slots)].copy_(t, non_blocking=True)
+        return out[: len(slots)]
+    return t.to(device) if device is not None else t

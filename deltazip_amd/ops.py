@@ -1,0 +1,276 @@
+"""Operator layer: the reference's delta ops, backed by the HIP kernels in libdz_amd.so.
+
+Mirrors
+  serving/vllm/delta/deltazip_marlin.py:10-19   apply_delta(x, qweight_stacked, scales_stacked,
+                                                meta_stacked, indices, base_weight) -> y
+  serving/vllm/delta/deltazip.py:14-77          add_delta / add_delta_slice (in-place y +=)
+of eth-easl/deltazip.  Tensor names and roles are the reference's; the bit layout inside
+`qweight`/`meta` is this project's native gfx950 layout (see csrc/dz_layout.h), produced from the
+reference's GPTQ-style tensors by `repack_gptq_to_native`.
+
+PyTorch is used for device memory and streams only; all arithmetic happens in the library.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from . import _lib
+
+MAX_TOKENS_FUSED = 128
+
+# ---------------------------------------------------------------------------------------------
+# layout helpers
+# ---------------------------------------------------------------------------------------------
+
+
+def native_sizes(K: int, N: int, bits: int, group_size: int = -1) -> Tuple[int, int, int]:
+    """(codes_bytes, meta_bytes, scales_bytes) of one delta in the native layout."""
+    cb, mb, sb = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    _lib.check(_lib.lib().dz_native_sizes(K, N, bits, group_size, C.byref(cb), C.byref(mb), C.byref(sb)),
+               "dz_native_sizes")
+    return cb.value, mb.value, sb.value
+
+
+def stacked_shapes(K: int, N: int, bits: int, group_size: int = -1):
+    """Shapes (without the leading slot dimension) of the three stacked tensors, following
+    layers_marlin.py:311-333: qweight [K/(pf*4), 2N] int32, meta [N, K/16] int16, scales [G, N]."""
+    native_sizes(K, N, bits, group_size)  # validates
+    pf = 32 // bits
+    g = 1 if group_size in (-1, K) else K // group_size
+    return (K // (pf * 4), 2 * N), (N, K // 16), (g, N)
+
+
+def repack_gptq_to_native(qweight: torch.Tensor, qzeros: torch.Tensor, scales: torch.Tensor,
+                          g_idx: Optional[torch.Tensor], bits: int):
+    """GPTQ-style tensors of one delta (as QuantLinear.pack writes them,
+    deltazip/nn_modules/qlinear_cuda.py:144-244) -> (qweight, meta, scales) CPU tensors in the
+    native layout, shaped as `stacked_shapes` says.  Host work, done once per delta; stands where
+    the reference calls its checkpoint converter (deltazip/utils/converter.py:13-101)."""
+    if bits not in (2, 4):
+        raise NotImplementedError("Only 2 and 4 bits are supported.")
+    qweight = qweight.detach().cpu().contiguous()
+    qzeros = qzeros.detach().cpu().contiguous()
+    scales = scales.detach().cpu().contiguous()
+    if qweight.dtype != torch.int32 or qzeros.dtype != torch.int32 or scales.dtype != torch.float16:
+        raise ValueError("qweight/qzeros must be int32 and scales float16")
+    pf = 32 // bits
+    K, N = qweight.shape[0] * pf, qweight.shape[1]
+    G = scales.shape[0]
+    if scales.shape != (G, N) or qzeros.shape != (G, N // pf) or K % G:
+        raise ValueError("inconsistent qzeros/scales shapes")
+    group_size = -1 if G == 1 else K // G
+    gi = None
+    if g_idx is not None:
+        gi = g_idx.detach().cpu().to(torch.int32).contiguous()
+        if gi.numel() != K:
+            raise ValueError("g_idx must have K entries")
+    (qs, ms, ss) = stacked_shapes(K, N, bits, group_size)
+    out_q = torch.empty(qs, dtype=torch.int32)
+    out_m = torch.empty(ms, dtype=torch.int16)
+    out_s = torch.empty(ss, dtype=torch.float16)
+    rc = _lib.lib().dz_repack_2of4(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(),
+                                   gi.data_ptr() if gi is not None else None, K, N, bits, group_size,
+                                   out_q.data_ptr(), out_m.data_ptr(), out_s.data_ptr())
+    _lib.check(rc, "dz_repack_2of4")
+    return out_q, out_m, out_s
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("tensors must live on the GPU (there is no CPU implementation)")
+
+
+def dequant(qweight: torch.Tensor, meta: torch.Tensor, scales: torch.Tensor, K: int, N: int,
+            bits: int) -> torch.Tensor:
+    """One native delta -> fp16 [N, K] on the GPU; bit-exact with QuantLinear.unpack
+    (deltazip/nn_modules/qlinear_cuda.py:246-329)."""
+    _need_cuda(qweight, meta, scales)
+    G = scales.numel() // N
+    out = torch.empty((N, K), dtype=torch.float16, device=qweight.device)
+    rc = _lib.lib().dz_dequant(qweight.data_ptr(), meta.data_ptr(), scales.data_ptr(), K, N, bits,
+                               -1 if G == 1 else K // G, out.data_ptr(), _stream())
+    _lib.check(rc, "dz_dequant")
+    return out
+
+
+def merge(base_weight: torch.Tensor, qweight, meta, scales, bits: int) -> torch.Tensor:
+    """W_base + dequant(delta) as fp16 [N, K] (deltazip/utils/generate.py:9-20 at fp16 storage)."""
+    _need_cuda(base_weight, qweight, meta, scales)
+    N, K = base_weight.shape
+    G = scales.numel() // N
+    out = torch.empty_like(base_weight)
+    rc = _lib.lib().dz_merge(base_weight.data_ptr(), qweight.data_ptr(), meta.data_ptr(),
+                             scales.data_ptr(), K, N, bits, -1 if G == 1 else K // G, out.data_ptr(),
+                             _stream())
+    _lib.check(rc, "dz_merge")
+    return out
+
+
+def segment(indices: torch.Tensor, num_slots: int):
+    """(perm [T] int32, seg_off [S+2] int32): tokens grouped by delta id, id -1 first."""
+    _need_cuda(indices)
+    if indices.dtype != torch.int64:
+        raise ValueError("indices must be int64")
+    T = indices.numel()
+    perm = torch.empty(T, dtype=torch.int32, device=indices.device)
+    off = torch.empty(num_slots + 2, dtype=torch.int32, device=indices.device)
+    _lib.check(_lib.lib().dz_segment(indices.data_ptr(), T, num_slots, perm.data_ptr(), off.data_ptr(),
+                                     _stream()), "dz_segment")
+    return perm, off
+
+
+# ---------------------------------------------------------------------------------------------
+# workspace: zero-filled once per device, reused by every call on that device
+# ---------------------------------------------------------------------------------------------
+_workspaces: Dict[int, torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, T: int, K: int, N: int) -> torch.Tensor:
+    need = _lib.lib().dz_workspace_bytes(T, K, N)
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    ws = _workspaces.get(idx)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[idx] = ws
+    return ws
+
+
+def workspace_status(device=None) -> int:
+    """Status word of the device workspace (bit 0: a delta id outside [-1, S) was seen and treated
+    as -1).  Synchronises; meant for debugging and tests."""
+    idx = torch.cuda.current_device() if device is None else torch.device(device).index
+    ws = _workspaces.get(idx)
+    if ws is None:
+        return 0
+    return int(ws[:4].view(torch.int32).item())
+
+
+# ---------------------------------------------------------------------------------------------
+# the ops
+# ---------------------------------------------------------------------------------------------
+
+
+def _infer(qweight_stacked, scales_stacked, N: int):
+    """(K, bits, group_size, S) from the stacked tensors' shapes."""
+    S = qweight_stacked.shape[0]
+    words = qweight_stacked[0].numel()
+    G = scales_stacked[0].numel() // N
+    return S, words, G
+
+
+def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qweight_stacked,
+                       scales_stacked, meta_stacked, indices: torch.Tensor, *, bits: int,
+                       out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+    """y = x @ W_base^T + x @ dequant(delta[indices])^T.  `out` may be a column slice of a wider
+    tensor (last-dim stride 1); with accumulate=True the result is added to it."""
+    _need_cuda(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices)
+    if x.dtype != torch.float16:
+        raise ValueError("x must be float16")
+    if indices.dtype != torch.int64:
+        raise ValueError("indices must be int64")
+    if bits not in (2, 4):
+        raise NotImplementedError("Only 2 and 4 bits are supported.")
+    K = x.shape[-1]
+    x2 = x.reshape(-1, K)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    T = x2.shape[0]
+    indices = indices.reshape(-1)
+    if indices.numel() != T or not indices.is_contiguous():
+        raise ValueError("indices must be a contiguous vector with one entry per token")
+    S = qweight_stacked.shape[0]
+    N = scales_stacked.shape[-1]
+    if base_weight is not None:
+        if base_weight.dtype != torch.float16 or tuple(base_weight.shape) != (N, K) or not base_weight.is_contiguous():
+            raise ValueError("base_weight must be a contiguous float16 [N, K] tensor")
+    G = scales_stacked[0].numel() // N
+    group_size = -1 if G == 1 else K // G
+    cb, mb, sb = native_sizes(K, N, bits, group_size)
+    if (qweight_stacked[0].numel() * qweight_stacked.element_size() != cb
+            or meta_stacked[0].numel() * meta_stacked.element_size() != mb
+            or not qweight_stacked.is_contiguous() or not meta_stacked.is_contiguous()
+            or not scales_stacked.is_contiguous() or scales_stacked.dtype != torch.float16):
+        raise ValueError("stacked delta tensors do not match the native layout for these sizes")
+    if out is None:
+        if accumulate:
+            raise ValueError("accumulate needs an output tensor")
+        out = torch.empty((T, N), dtype=torch.float16, device=x.device)
+    else:
+        if out.dtype != torch.float16 or out.dim() != 2 or out.shape != (T, N) or out.stride(1) != 1:
+            raise ValueError("out must be float16 [T, N] with unit column stride")
+    ldy = out.stride(0)
+    if T > MAX_TOKENS_FUSED:
+        from .prefill import multi_delta_linear_prefill
+        return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
+                                          indices, bits=bits, out=out, accumulate=accumulate)
+    ws = _workspace(x.device, T, K, N)
+    rc = _lib.lib().dz_multi_delta_linear(
+        x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
+        qweight_stacked.data_ptr(), meta_stacked.data_ptr(), scales_stacked.data_ptr(),
+        indices.data_ptr(), out.data_ptr(), T, K, N, S, bits, group_size, 1 if accumulate else 0, ldy,
+        ws.data_ptr(), ws.numel(), _stream())
+    _lib.check(rc, "dz_multi_delta_linear")
+    return out
+
+
+def _bits_from_shapes(qweight_stacked: torch.Tensor, K: int, N: int) -> int:
+    words = qweight_stacked[0].numel()
+    bits = words * 64 // (K * N)  # words = K*N*bits/64
+    if bits not in (2, 4) or words * 64 != K * N * bits:
+        raise ValueError("cannot infer the bit width from qweight_stacked")
+    return bits
+
+
+def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: torch.Tensor,
+                meta_stacked: torch.Tensor, indices: torch.Tensor, base_weight: torch.Tensor) -> torch.Tensor:
+    """Drop-in for serving/vllm/delta/deltazip_marlin.py:10-19.  Returns a new [T, N] tensor;
+    indices == -1 selects the base weight only."""
+    N, K = base_weight.shape
+    bits = _bits_from_shapes(qweight_stacked, K, N)
+    y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits)
+    return y.view(*x.shape[:-1], N)
+
+
+def add_delta(y: torch.Tensor, x: torch.Tensor, qweight: torch.Tensor, qzeros, scales: torch.Tensor,
+              g_idx, indices: torch.Tensor, meta: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Drop-in for serving/vllm/delta/deltazip.py:14-37: y[i] += x[i] @ dequant(W[indices[i]])^T,
+    in place.  `qzeros` and `g_idx` are accepted for signature compatibility and unused: the native
+    layout is symmetric with g_idx = k // group_size (checked when the delta was repacked)."""
+    if meta is None:
+        raise ValueError("meta (2:4 positions) is required")
+    K = x.shape[-1]
+    N = scales.shape[-1]
+    bits = _bits_from_shapes(qweight, K, N)
+    y2 = y.view(-1, y.shape[-1])
+    multi_delta_linear(x, None, qweight, scales, meta, indices, bits=bits, out=y2, accumulate=True)
+    return y
+
+
+def add_delta_slice(y: torch.Tensor, x: torch.Tensor, qweight, qzeros, scales, g_idx, indices,
+                    scale: float, y_offset: int, y_slice_size: int, *, buffer=None,
+                    meta: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Drop-in for serving/vllm/delta/deltazip.py:40-77: as add_delta, into the column slice
+    y[:, y_offset : y_offset + y_slice_size].  `scale` is ignored, as it is by the reference."""
+    if meta is None:
+        raise ValueError("meta (2:4 positions) is required")
+    K = x.shape[-1]
+    N = scales.shape[-1]
+    if N != y_slice_size:
+        raise ValueError("y_slice_size must equal the delta's output features")
+    bits = _bits_from_shapes(qweight, K, N)
+    y2 = y.view(-1, y.shape[-1])[:, y_offset:y_offset + y_slice_size]
+    multi_delta_linear(x, None, qweight, scales, meta, indices, bits=bits, out=y2, accumulate=True)
+    return y
+
+
+def set_ksplit(nsplit: int) -> None:
+    """Benchmark hook: force the number of K chunks of the fused kernel (0 = automatic)."""
+    _lib.lib().dz_set_ksplit(int(nsplit))

@@ -1,0 +1,114 @@
+/*
+ * dz_amd.h -- C ABI of the MI355X (gfx950) multi-delta linear layer.
+ *
+ *   y[t, :] = x[t, :] @ W_base^T  +  (ids[t] >= 0 ?  x[t, :] @ dequant(delta[ids[t]])^T : 0)
+ *
+ * Every delta is 2:4 sparse along the input dimension, quantised symmetrically to 2 or 4 bits
+ * with fp16 scales (per output channel, or per (channel, K-group)).  All pointers are raw
+ * device pointers unless a parameter is documented as host memory; the caller owns all
+ * memory.  Functions return 0 on success or a negative DZ_E* code; dz_strerror() names it.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).  Launches are
+ * asynchronous on that stream.  No function allocates device memory.
+ *
+ * Reference interfaces these entry points stand in for (paths relative to the
+ * eth-easl/deltazip tree):
+ *   serving/vllm/delta/deltazip_marlin.py:10-19    apply_delta -> sbmm_4bit_2_4_native
+ *   serving/vllm/delta/deltazip.py:14-77           add_delta / add_delta_slice -> ibmm_sparse_marlin
+ *   serving/vllm/delta/quant_linears/quant_linear_naive.py:35-96   QuantLinear.forward/from_tensors
+ *   deltazip/nn_modules/qlinear_cuda.py:246-329    QuantLinear.unpack (dequantisation)
+ *   deltazip/utils/converter.py:13-101             GPTQ layout -> kernel layout conversion
+ */
+#ifndef DZ_AMD_H
+#define DZ_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DZ_OK            0
+#define DZ_EINVAL       -1   /* bad argument (null pointer, negative size)                  */
+#define DZ_ESHAPE       -2   /* shape not supported: K % 256, N % 32, ldy % 4, T range      */
+#define DZ_EBITS        -3   /* bits not in {2, 4}                                         */
+#define DZ_EGROUP       -4   /* group_size not -1/K or a multiple of 64 dividing K          */
+#define DZ_ENOT24       -5   /* repack: a group of 4 holds more than 2 non-zero-point codes */
+#define DZ_EZERO        -6   /* repack: zero-point differs from 2^(bits-1)                  */
+#define DZ_EGIDX        -7   /* repack: g_idx is not k / group_size                         */
+#define DZ_EWORKSPACE   -8   /* workspace missing or too small                             */
+#define DZ_ELAUNCH      -9   /* the HIP runtime refused the launch                         */
+#define DZ_EALIGN      -10   /* pointer not aligned as required                            */
+
+#define DZ_MAX_TOKENS_FUSED 128   /* largest T the fused decode kernel takes in one launch   */
+
+/* Library version (major*10000 + minor*100 + patch). */
+int dz_version(void);
+
+/* Static, human readable text for a return code. */
+const char* dz_strerror(int code);
+
+/* Byte sizes of one delta in the native layout (per slot strides of the stacked tensors).
+ * Stands in for the shape arithmetic of BaseLayerWithDelta.create_delta_weights
+ * (serving/vllm/delta/layers_marlin.py:311-333). */
+int dz_native_sizes(int K, int N, int bits, int group_size,
+                    size_t* codes_bytes, size_t* meta_bytes, size_t* scales_bytes);
+
+/* HOST function, host pointers.  Converts one delta from the reference's GPTQ-style packing
+ * (qweight [K*bits/32, N] int32, qzeros [G, N*bits/32] int32 holding zero-1, scales [G, N] fp16,
+ * g_idx [K] int32; deltazip/nn_modules/qlinear_cuda.py:144-244) into the native layout
+ * (codes, meta, scales) consumed by the kernels.  Takes the role of
+ * deltazip/utils/converter.py:13-101 (the conversion the reference delegates to triteia). */
+int dz_repack_2of4(const int32_t* qweight, const int32_t* qzeros, const uint16_t* scales,
+                   const int32_t* g_idx, int K, int N, int bits, int group_size,
+                   void* out_codes, void* out_meta, void* out_scales);
+
+/* Dequantise one native delta to fp16, out[n * K + k] (row-major [N, K]).  Bit-exact with
+ * QuantLinear.unpack (deltazip/nn_modules/qlinear_cuda.py:246-329): half(float(scale)*(q-zero)). */
+int dz_dequant(const void* codes, const void* meta, const void* scales,
+               int K, int N, int bits, int group_size, uint16_t* out, void* stream);
+
+/* out[n*K+k] = w_base[n*K+k] + dequant(delta)[n, k], the addition done in fp32 and rounded once
+ * to fp16 (the reference's merge, deltazip/utils/generate.py:9-20, at fp16 storage). */
+int dz_merge(const uint16_t* w_base, const void* codes, const void* meta, const void* scales,
+             int K, int N, int bits, int group_size, uint16_t* out, void* stream);
+
+/* Group tokens by delta id: perm[T] lists token indices sorted by id (stable; id -1 first),
+ * seg_off[S + 2] are the offsets of the segments for id = -1, 0, ..., S-1 in perm.
+ * Ids outside [-1, S) are treated as -1.  (The reference's scheduler sorts the batch by delta
+ * id, serving/vllm/core/scheduler.py:101-104; this makes the op independent of that.) */
+int dz_segment(const int64_t* indices, int T, int S, int32_t* perm, int32_t* seg_off, void* stream);
+
+/* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
+ * zero-filled once before first use; calls leave it ready for the next call.  Calls that share
+ * a workspace must be ordered on one stream. */
+size_t dz_workspace_bytes(int T, int K, int N);
+
+/* The layer.  x [T, K] fp16 row-major; w_base [N, K] fp16 row-major or NULL (delta only);
+ * codes/meta/scales: S slots of one native delta each, slot strides as dz_native_sizes reports;
+ * indices [T] int64, -1 = base only, read on the device at execution time; y [T, ldy] fp16,
+ * columns 0..N-1 written.  accumulate = 0: y = result; 1: y += result (fp32 add, one rounding).
+ * Stands in for sbmm_4bit_2_4_native / ibmm_sparse_marlin at the call sites listed above.
+ * T <= DZ_MAX_TOKENS_FUSED uses the single fused kernel; larger T runs the segment-wise
+ * merge + matrix-core GEMM path and needs prefill workspace (dz_workspace_bytes covers it). */
+int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
+                          const void* codes_stacked, const void* meta_stacked,
+                          const void* scales_stacked, const int64_t* indices, uint16_t* y,
+                          int T, int K, int N, int S, int bits, int group_size,
+                          int accumulate, int ldy, void* workspace, size_t workspace_bytes,
+                          void* stream);
+
+/* Dense fp16 GEMM on the matrix cores: y[T, ldy] (+)= x[T, K] @ w[N, K]^T, fp32 accumulation.
+ * Stands in for the base product of LinearMethodBase.apply_weights
+ * (serving/vllm/model_executor/layers/linear.py:85-96) at prefill sizes. */
+int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
+                int accumulate, int ldy, void* stream);
+
+/* Tuning hook used by the benchmark: override the split of K across workgroups of the fused
+ * kernel (0 = automatic). */
+void dz_set_ksplit(int nsplit);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DZ_AMD_H */

@@ -1,0 +1,433 @@
+"""CPU oracle for the multi-delta linear layer.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, on the CPU and in numpy (+ torch CPU matmul), the algorithm that
+eth-easl/deltazip runs for  y = x @ W_base.T + x @ dequant(delta[id(x)]).T .  It exists to
+check the HIP kernels; only tests, the smoke check and the benchmark's CPU-baseline leg may
+import it.  Nothing in the shipped package depends on it.
+
+Every function names the reference lines it follows (paths relative to the reference root).
+
+Pinning status (what independent evidence each function is checked against in tests/):
+  quantize, find_params_sym     closed forms + known answers computed by hand          (pinned)
+  prune_2of4_magnitude          brute force on tiny rows, group invariants             (pinned)
+  pack_gptq / unpack_gptq       single-bit probes, hand-packed words, round trips      (pinned)
+  dequant_gptq                  exhaustive fp16-scale sweep against exact rational math (pinned)
+  forward_ref                   per-token python loop, F.linear special cases          (pinned)
+  native layout functions       defined by this project; pinned by round trip through
+                                dequant_gptq
+The fused third-party kernel the reference calls on the serving path (triteia
+`sbmm_4bit_2_4_native`, un-vendored and un-pinned: scripts/install.sh:2, call site
+serving/vllm/delta/deltazip_marlin.py:18) cannot be inspected: its bit layout and rounding are
+"parity unpinned".  Parity is anchored on the reference's in-tree CPU-runnable path instead.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+# --------------------------------------------------------------------------------------
+# a1/a2: quantizer  (deltazip/core/quant.py)
+# --------------------------------------------------------------------------------------
+
+
+def quantize(x: np.ndarray, scale: np.ndarray, zero: np.ndarray, maxq: int) -> np.ndarray:
+    """deltazip/core/quant.py:9-18.  q = clamp(round(x/scale)+zero, 0, maxq); returns
+    scale*(q-zero).  torch.round is round-half-to-even, as is np.rint.  fp32 throughout."""
+    x = x.astype(np.float32)
+    q = np.clip(np.rint(x / scale) + zero, 0, maxq).astype(np.float32)
+    return (scale * (q - zero)).astype(np.float32)
+
+
+def quantize_codes(x, scale, zero, maxq):
+    """Integer codes of `quantize` (the q before it is mapped back), uint8."""
+    x = x.astype(np.float32)
+    return np.clip(np.rint(x / scale) + zero, 0, maxq).astype(np.uint8)
+
+
+def find_params_sym(w: np.ndarray, bits: int, group_size: int = -1):
+    """Symmetric per-output-row (optionally per (row, K-group)) scale and zero.
+
+    deltazip/core/quant.py:48-130 with perchannel=True, sym=True, mse=False, weight=True
+    (the configuration deltazip/modeling/_base.py:399-406 uses).  `w` is [N, K] fp32.
+    Returns (scale [N, G] fp32, zero [N, G] fp32) with G = 1 for group_size == -1.
+
+    The reference computes the parameters on the un-pruned delta (core/sparsegpt.py:64-66).
+    Grouping along K is a format-compatible extension (the reference's g_idx mechanism); each
+    group is treated exactly like a full row is by the reference.
+    """
+    w = w.astype(np.float32)
+    n, k = w.shape
+    g = k if group_size in (-1, k) else group_size
+    assert k % g == 0
+    maxq = 2**bits - 1
+    wg = w.reshape(n, k // g, g)
+    xmin = np.minimum(wg.min(axis=2), 0.0).astype(np.float32)       # quant.py:69
+    xmax = np.maximum(wg.max(axis=2), 0.0).astype(np.float32)       # quant.py:70
+    xmax = np.maximum(np.abs(xmin), xmax)                           # quant.py:73
+    neg = xmin < 0
+    xmin = np.where(neg, -xmax, xmin)                               # quant.py:74-76
+    both0 = (xmin == 0) & (xmax == 0)                               # quant.py:77-79
+    xmin = np.where(both0, -1.0, xmin).astype(np.float32)
+    xmax = np.where(both0, +1.0, xmax).astype(np.float32)
+    scale = ((xmax - xmin) / np.float32(maxq)).astype(np.float32)   # quant.py:81
+    zero = np.full_like(scale, (maxq + 1) / 2)                      # quant.py:83
+    return scale, zero
+
+
+# --------------------------------------------------------------------------------------
+# a3: 2:4 mask rule (deltazip/core/sparsegpt.py:117-135 with H = I)
+# --------------------------------------------------------------------------------------
+
+
+def prune_2of4_magnitude(w: np.ndarray) -> np.ndarray:
+    """Boolean keep-mask [N, K]: in every aligned group of 4 along K keep the 2 entries of
+    largest |w|.  core/sparsegpt.py:123-125 prunes the `prunen`=2 entries with the smallest
+    w^2/diag(Hinv)^2 in each group of `prunem`=4; with an identity Hessian that is the 2
+    smallest |w|.  torch.topk leaves ties unspecified; here ties keep the lower column index.
+    """
+    n, k = w.shape
+    assert k % 4 == 0
+    a = np.abs(w.astype(np.float32)).reshape(n, k // 4, 4)
+    # rank of each entry inside its group under (larger |w| first, lower index first on ties)
+    rank = np.zeros(a.shape, dtype=np.int8)
+    for i in range(4):
+        for j in range(4):
+            if i == j:
+                continue
+            ahead = (a[:, :, j] > a[:, :, i]) if j > i else (a[:, :, j] >= a[:, :, i])
+            rank[:, :, i] += ahead
+    return (rank < 2).reshape(n, k)
+
+
+def compress_delta(delta32: np.ndarray, bits: int, group_size: int = -1):
+    """delta [N, K] fp32 -> (codes [K, N] uint8, scales16 [G, N] fp16, zeros [G, N] int, keep).
+
+    Order of operations follows core/sparsegpt.py:64-66 (parameters from the un-pruned
+    delta), :123-135 (pruned entries are set to 0 and then quantized, so their code is the
+    zero-point and they dequantize to exactly 0).
+    """
+    n, k = delta32.shape
+    maxq = 2**bits - 1
+    scale, zero = find_params_sym(delta32, bits, group_size)       # [N, G]
+    g = k // scale.shape[1]
+    keep = prune_2of4_magnitude(delta32)
+    wp = np.where(keep, delta32.astype(np.float32), np.float32(0))
+    scale_full = np.repeat(scale, g, axis=1)
+    zero_full = np.repeat(zero, g, axis=1)
+    codes = quantize_codes(wp, scale_full, zero_full, maxq)        # [N, K]
+    return (np.ascontiguousarray(codes.T), np.ascontiguousarray(scale.T.astype(np.float16)),
+            np.ascontiguousarray(zero.T.astype(np.int32)), keep)
+
+
+# --------------------------------------------------------------------------------------
+# a4: GPTQ-style packing (deltazip/nn_modules/qlinear_cuda.py:144-244)
+# --------------------------------------------------------------------------------------
+
+
+def pack_codes_gptq(codes: np.ndarray, zeros: np.ndarray, scales16: np.ndarray, bits: int):
+    """codes [K, N] uint8, zeros [G, N] int (true zero-points), scales16 [G, N] fp16 ->
+    (qweight [K/pf, N] int32, qzeros [G, N/pf] int32, scales [G, N] fp16, g_idx [K] int32).
+
+    qlinear_cuda.py:177-182: qweight[r, n] |= code[r*pf + j, n] << (bits*j), j = 0..pf-1.
+    qlinear_cuda.py:208-220: qzeros stores (zero - 1), packed along N the same way.
+    qlinear_cuda.py:81-86 / sparsegpt.py:161-162: g_idx[k] = k // group_size.
+    """
+    assert bits in (2, 4, 8)
+    k, n = codes.shape
+    pf = 32 // bits
+    assert k % pf == 0 and n % pf == 0
+    c = codes.astype(np.uint32).reshape(k // pf, pf, n)
+    qweight = np.zeros((k // pf, n), dtype=np.uint32)
+    for j in range(pf):
+        qweight |= c[:, j, :] << np.uint32(bits * j)
+    g = zeros.shape[0]
+    z = (zeros.astype(np.int64) - 1).astype(np.uint32).reshape(g, n // pf, pf)
+    qzeros = np.zeros((g, n // pf), dtype=np.uint32)
+    for j in range(pf):
+        qzeros |= (z[:, :, j] & np.uint32(2**bits - 1)) << np.uint32(bits * j)
+    group = k // g
+    g_idx = (np.arange(k) // group).astype(np.int32)
+    return qweight.view(np.int32), qzeros.view(np.int32), scales16.astype(np.float16), g_idx
+
+
+def pack_from_weights(w_deq: np.ndarray, scale: np.ndarray, zero: np.ndarray, bits: int):
+    """The reference's `QuantLinear.pack` starting, as it does, from the dequantized fp32
+    weights: intweight[k, n] = round((W[n, k] + zero*scale) / half(scale))
+    (qlinear_cuda.py:153-168; the division uses the fp16-rounded scale).  w_deq [N, K] fp32,
+    scale/zero [N, G] fp32.  Returns the same tuple as pack_codes_gptq."""
+    n, k = w_deq.shape
+    g = scale.shape[1]
+    group = k // g
+    scales_t = np.ascontiguousarray(scale.T).astype(np.float32)       # [G, N]
+    zeros_t = np.ascontiguousarray(zero.T).astype(np.float32)
+    scale_zeros = zeros_t * scales_t
+    scales16 = scales_t.astype(np.float16)
+    gi = np.arange(k) // group
+    num = w_deq.T.astype(np.float32) + scale_zeros[gi]                 # [K, N]
+    codes = np.rint(num / scales16[gi].astype(np.float32)).astype(np.int64)
+    codes = codes.astype(np.uint32).astype(np.uint8)
+    return pack_codes_gptq(codes, zeros_t.astype(np.int32), scales16, bits)
+
+
+def unpack_gptq(qweight: np.ndarray, qzeros: np.ndarray, bits: int):
+    """qlinear_cuda.py:250-264 / quant_linear_naive.py:43-58: shift right by bits*j, mask with
+    2^bits-1, zeros get +1.  Returns (codes [K, N] int8/int16, zeros [G, N] same dtype)."""
+    assert bits in (2, 4, 8)
+    pf = 32 // bits
+    mask = 2**bits - 1
+    dt = np.int16 if bits == 8 else np.int8
+    wf = (np.arange(pf) * bits).astype(np.uint32)
+    qw = qweight.view(np.uint32)
+    codes = ((qw[:, None, :] >> wf[None, :, None]) & np.uint32(mask)).astype(dt)
+    codes = codes.reshape(qw.shape[0] * pf, qw.shape[1])
+    qz = qzeros.view(np.uint32)
+    zeros = ((qz[:, :, None] >> wf[None, None, :]) & np.uint32(mask)).astype(dt) + dt(1)
+    zeros = zeros.reshape(qz.shape[0], qz.shape[1] * pf)
+    return codes, zeros
+
+
+# --------------------------------------------------------------------------------------
+# a5: dequantisation (qlinear_cuda.py:306-308, quant_linear_naive.py:65-67)
+# --------------------------------------------------------------------------------------
+
+
+def dequant_gptq(qweight, qzeros, scales16, g_idx, bits) -> np.ndarray:
+    """delta^T [K, N] fp16 = scales[g_idx] * (codes - zeros[g_idx]).
+
+    In the reference this is an fp16 tensor times an int8 tensor, which torch evaluates as
+    one correctly rounded fp16 product.  The integer factor has at most 5 significant bits and
+    the scale 11, so the fp32 product is exact and a single fp32->fp16 round-to-nearest-even
+    reproduces it; that is what is computed here."""
+    codes, zeros = unpack_gptq(qweight, qzeros, bits)
+    gi = g_idx.astype(np.int64)
+    m = (codes.astype(np.int32) - zeros[gi].astype(np.int32)).astype(np.float32)
+    s = scales16.astype(np.float16)[gi].astype(np.float32)
+    return (s * m).astype(np.float16)
+
+
+# --------------------------------------------------------------------------------------
+# a6/a7/a8: forward
+# --------------------------------------------------------------------------------------
+
+
+def forward_ref(x16: np.ndarray, w_base16, delta_t_list, ids: np.ndarray) -> np.ndarray:
+    """fp32 layer output [T, N].
+
+    Semantics of apply_delta (serving/vllm/delta/deltazip_marlin.py:10-19; per-token rule
+    spelled out at serving/vllm/delta/deltazip.py:24-30): token t uses W_base plus the delta
+    in slot ids[t], ids[t] == -1 meaning base only.  The weight is formed as the reference's
+    merge does, W = W_base + delta (deltazip/utils/generate.py:9-20), in fp32, and tokens are
+    grouped by id with one dense product per id, the reference's own idiom for this
+    (deltazip_marlin.py:44-53).  w_base16 may be None (delta-only, for the add_delta forms).
+    delta_t_list[d] is delta^T [K, N] fp16 as dequant_gptq returns it."""
+    x = torch.from_numpy(np.ascontiguousarray(x16).astype(np.float32))
+    t = x.shape[0]
+    n = (w_base16.shape[0] if w_base16 is not None else delta_t_list[0].shape[1])
+    y = torch.zeros((t, n), dtype=torch.float32)
+    wb = None if w_base16 is None else torch.from_numpy(np.ascontiguousarray(w_base16).astype(np.float32))
+    ids = np.asarray(ids).astype(np.int64)
+    for d in np.unique(ids):
+        sel = torch.from_numpy(np.nonzero(ids == d)[0])
+        if d >= 0:
+            w = torch.from_numpy(np.ascontiguousarray(delta_t_list[int(d)]).astype(np.float32)).t()
+            if wb is not None:
+                w = wb + w
+        else:
+            if wb is None:
+                continue
+            w = wb
+        y[sel] = x[sel] @ w.t()
+    return y.numpy()
+
+
+def forward_token_loop(x16, w_base16, delta_t_list, ids) -> np.ndarray:
+    """Per-token loop in float64: the independent check for forward_ref, shaped like the
+    reference's multi-adapter kernel test (serving/tests/lora/test_punica.py:18-42)."""
+    t = x16.shape[0]
+    n = w_base16.shape[0]
+    y = np.zeros((t, n), dtype=np.float64)
+    for i in range(t):
+        xi = x16[i].astype(np.float64)
+        y[i] = w_base16.astype(np.float64) @ xi
+        if ids[i] >= 0:
+            y[i] += xi @ delta_t_list[int(ids[i])].astype(np.float64)
+    return y
+
+
+def forward_naive_fp16(x16, w_base16, delta_t_list, ids) -> np.ndarray:
+    """The reference's fp16 serving arithmetic (quant_linear_naive.py:80: matmul(x.half(),
+    W) in fp16) added to an fp16 base product.  Reported beside the fp32 result, not gated."""
+    x = torch.from_numpy(np.ascontiguousarray(x16))
+    wb = torch.from_numpy(np.ascontiguousarray(w_base16))
+    y = (x.float() @ wb.float().t()).half()
+    for i, d in enumerate(ids):
+        if d >= 0:
+            dt = torch.from_numpy(np.ascontiguousarray(delta_t_list[int(d)]))
+            y[i] = y[i] + (x[i].float() @ dt.float()).half()
+    return y.numpy()
+
+
+def rel_err(y, y_ref) -> float:
+    """max |y - y_ref| / max(|y_ref|, 1e-3 * max|y_ref|): the layer-output parity metric."""
+    y = np.asarray(y, dtype=np.float64)
+    y_ref = np.asarray(y_ref, dtype=np.float64)
+    eps = 1e-3 * np.abs(y_ref).max()
+    return float(np.max(np.abs(y - y_ref) / np.maximum(np.abs(y_ref), eps)))
+
+
+# --------------------------------------------------------------------------------------
+# native gfx950 layout (defined by this project)
+# --------------------------------------------------------------------------------------
+# Tiles: an "n-pair" is 32 output rows (two 16-row fragments), a "k-block" is 256 input
+# columns (four 64-column steps).  One fragment = 16 rows x 64 columns; lane la = 16*ga + i of
+# a 64-lane wavefront owns row i and the four aligned groups-of-4 starting at
+#     k0(ga, p) = 16*(ga & 1) + 32*(ga >> 1) + 8*(p >> 1) + 4*(p & 1),   p = 0..3
+# inside the step.  Each group contributes its two kept elements (ascending position): element
+# e = 2p + w.  This is the operand order of the sparse matrix instruction
+# v_smfmac_f32_16x16x64_f16 when the dense operand's 16 per-lane values are taken as columns
+# 8*gb + (eb & 7) + 32*(eb >> 3).
+#   meta  uint32 [N/32][K/256][64 lanes][4 steps]: bits [16*s + 2*e, +2) = position (0..3) of
+#         element e of fragment (row-tile 2*np + s, step 4*kb + j).
+#   codes 2-bit uint32 [N/32][K/256][64][4]: word j; for s in 0..1, m in 0..3, t = 4*s + m:
+#         bits [2t, 2t+2) = code of element 2m, bits [16+2t, 16+2t+2) = code of element 2m+1.
+#   codes 4-bit uint32 [N/32][K/256][2][64][4]: half hf covers steps 2*hf, 2*hf+1; word
+#         w = 2*(j & 1) + s; bits [4m, 4m+4) = element 2m, bits [16+4m, 16+4m+4) = element 2m+1.
+#   scales fp16 [G][N] unchanged.
+
+
+def _frag_group_k0():
+    ga = np.arange(4)[:, None]
+    p = np.arange(4)[None, :]
+    return 16 * (ga & 1) + 32 * (ga >> 1) + 8 * (p >> 1) + 4 * (p & 1)   # [ga, p]
+
+
+def repack_native(qweight, qzeros, scales16, g_idx, bits):
+    """GPTQ layout -> native (codes uint32, meta uint32, scales fp16).  Raises ValueError when
+    the input is not 2:4 sparse, has a zero-point other than 2^(bits-1), or a g_idx other than
+    k // group_size."""
+    if bits not in (2, 4):
+        raise ValueError("native layout supports 2 and 4 bits")
+    codes, zeros = unpack_gptq(qweight, qzeros, bits)        # [K, N], [G, N]
+    k, n = codes.shape
+    if k % 256 or n % 32:
+        raise ValueError("native layout needs K % 256 == 0 and N % 32 == 0")
+    zp = 2 ** (bits - 1)
+    if not np.all(zeros == zp):
+        raise ValueError("only the symmetric zero-point 2^(bits-1) is supported")
+    g = scales16.shape[0]
+    if not np.array_equal(np.asarray(g_idx), np.arange(k) // (k // g)):
+        raise ValueError("g_idx must be k // group_size")
+    c = codes.T.astype(np.int32).reshape(n, k // 4, 4)        # [N, groups, 4]
+    nz = c != zp
+    if np.any(nz.sum(axis=2) > 2):
+        raise ValueError("input is not 2:4 sparse")
+    # kept positions: the non-zero-point entries, completed with the lowest free positions
+    pos = np.arange(4)[None, None, :]
+    key = np.where(nz, pos, pos + 4)                           # non-zero first, by position
+    order = np.sort(key, axis=2)[:, :, :2] % 4                 # two kept positions
+    order = np.sort(order, axis=2)                             # ascending position
+    kept = np.take_along_axis(c, order, axis=2)                # [N, groups, 2]
+    np_, nkb = n // 32, k // 256
+    k0 = _frag_group_k0()                                      # [ga, p]
+    # index arrays over (np, s, i, kb, j, ga, p)
+    s_ = np.arange(2); i_ = np.arange(16); j_ = np.arange(4)
+    meta = np.zeros((np_, nkb, 64, 4), dtype=np.uint32)
+    if bits == 2:
+        out = np.zeros((np_, nkb, 64, 4), dtype=np.uint32)
+    else:
+        out = np.zeros((np_, nkb, 2, 64, 4), dtype=np.uint32)
+    rows = (np.arange(np_)[:, None, None] * 32 + s_[None, :, None] * 16 + i_[None, None, :])  # [np,s,i]
+    for ga in range(4):
+        for p in range(4):
+            for j in range(4):
+                grp = (np.arange(nkb) * 256 + 64 * j + k0[ga, p]) // 4          # [kb]
+                pos2 = order[rows[:, :, :, None], grp[None, None, None, :]]     # [np,s,i,kb,2]
+                val2 = kept[rows[:, :, :, None], grp[None, None, None, :]]
+                for s in range(2):
+                    la = 16 * ga + i_
+                    for w in range(2):
+                        e = 2 * p + w
+                        pv = pos2[:, s, :, :, w].transpose(0, 2, 1).astype(np.uint32)  # [np,kb,i]
+                        cv = val2[:, s, :, :, w].transpose(0, 2, 1).astype(np.uint32)
+                        meta[:, :, la, j] |= pv << np.uint32(16 * s + 2 * e)
+                        m = e // 2
+                        if bits == 2:
+                            t = 4 * s + m
+                            out[:, :, la, j] |= cv << np.uint32(2 * t + 16 * (e & 1))
+                        else:
+                            out[:, :, j // 2, la, 2 * (j & 1) + s] |= cv << np.uint32(4 * m + 16 * (e & 1))
+    return out, meta, scales16.astype(np.float16).copy()
+
+
+def dequant_native(codes, meta, scales16, k, n, bits) -> np.ndarray:
+    """native -> delta [N, K] fp16 (note: [N, K], the transpose of dequant_gptq's output)."""
+    zp = 2 ** (bits - 1)
+    np_, nkb = n // 32, k // 256
+    g = scales16.shape[0]
+    group = k // g
+    out = np.zeros((n, k), dtype=np.float16)
+    k0 = _frag_group_k0()
+    i_ = np.arange(16)
+    sc = scales16.astype(np.float32)                          # [G, N]
+    for ga in range(4):
+        la = 16 * ga + i_
+        for p in range(4):
+            for j in range(4):
+                for s in range(2):
+                    for w in range(2):
+                        e = 2 * p + w
+                        pos = (meta[:, :, la, j] >> np.uint32(16 * s + 2 * e)) & np.uint32(3)   # [np,kb,i]
+                        m = e // 2
+                        if bits == 2:
+                            cv = (codes[:, :, la, j] >> np.uint32(2 * (4 * s + m) + 16 * (e & 1))) & np.uint32(3)
+                        else:
+                            cv = (codes[:, :, j // 2, la, 2 * (j & 1) + s] >> np.uint32(4 * m + 16 * (e & 1))) & np.uint32(15)
+                        rows = (np.arange(np_)[:, None, None] * 32 + 16 * s + i_[None, None, :])
+                        rows = np.broadcast_to(rows, pos.shape)
+                        cols = (np.arange(nkb)[None, :, None] * 256 + 64 * j + k0[ga, p]) + pos.astype(np.int64)
+                        val = (sc[cols // group, rows] * (cv.astype(np.float32) - zp)).astype(np.float16)
+                        # a later kept element that dequantises to 0 must not erase an earlier value:
+                        # positions are distinct within a group, so plain assignment is safe.
+                        out[rows, cols] = val
+    return out
+
+
+# --------------------------------------------------------------------------------------
+# seeded synthetic inputs for the benchmark configurations
+# --------------------------------------------------------------------------------------
+
+
+def _randn(shape, seed):
+    g = torch.Generator(device="cpu").manual_seed(int(seed))
+    return torch.randn(shape, generator=g, dtype=torch.float32).numpy()
+
+
+def make_base(n, k, seed):
+    return (_randn((n, k), seed) * np.float32(0.02)).astype(np.float16)
+
+
+def make_delta(n, k, sigma, bits, group_size, seed):
+    """Returns dict with GPTQ-format tensors of one synthetic 2:4 delta."""
+    d = _randn((n, k), seed) * np.float32(sigma)
+    codes, scales16, zeros, keep = compress_delta(d, bits, group_size)
+    qweight, qzeros, scales, g_idx = pack_codes_gptq(codes, zeros, scales16, bits)
+    return dict(qweight=qweight, qzeros=qzeros, scales=scales, g_idx=g_idx, bits=bits,
+                delta32=d, keep=keep, codes=codes)
+
+
+def make_x(t, k, seed):
+    return _randn((t, k), seed).astype(np.float16)
+
+
+def make_ids(kind, t, n_deltas, seed):
+    g = torch.Generator(device="cpu").manual_seed(int(seed))
+    if kind == "single":
+        return np.zeros(t, dtype=np.int64)
+    if kind == "uniform":
+        return torch.randint(0, n_deltas, (t,), generator=g).numpy().astype(np.int64)
+    if kind == "zipf":
+        p = torch.arange(1, n_deltas + 1, dtype=torch.float64) ** -1.5
+        return torch.multinomial(p / p.sum(), t, replacement=True, generator=g).numpy().astype(np.int64)
+    if kind == "blocks":
+        return np.repeat(np.arange(n_deltas), t // n_deltas).astype(np.int64)
+    raise ValueError(kind)

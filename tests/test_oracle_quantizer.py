@@ -1,0 +1,90 @@
+"""Pins the oracle's quantizer and 2:4 mask (reference: deltazip/core/quant.py:9-18, 48-130;
+deltazip/core/sparsegpt.py:117-135 with H = I) against closed forms and brute force."""
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import dz_oracle as o
+
+
+def test_closed_form_4bit():
+    row = np.array([[0.003, -0.001, 0.0005, -0.0029]], dtype=np.float32)
+    scale, zero = o.find_params_sym(row, 4)
+    assert zero[0, 0] == 8
+    assert scale[0, 0] == np.float32(np.float32(0.006) / np.float32(15))      # 2*max|row|/15
+    # 0.003/scale = 7.5 -> half-to-even 8 -> +8 = 16 -> clamp 15
+    assert o.quantize_codes(row, scale, zero, 15).tolist() == [[15, 5, 9, 1]]
+
+
+def test_closed_form_2bit():
+    row = np.array([[0.003, -0.001, 0.0005, -0.0029]], dtype=np.float32)
+    scale, zero = o.find_params_sym(row, 2)
+    assert zero[0, 0] == 2 and scale[0, 0] == np.float32(np.float32(0.006) / np.float32(3))
+    codes = o.quantize_codes(row, scale, zero, 3)
+    assert codes.tolist() == [[3, 2, 2, 1]]
+    deq = o.quantize(row, scale, zero, 3)
+    assert np.allclose(deq, [[scale[0, 0], 0, 0, -scale[0, 0]]])
+
+
+def test_all_zero_row_uses_unit_range():
+    scale, zero = o.find_params_sym(np.zeros((1, 8), np.float32), 4)
+    assert scale[0, 0] == np.float32(2.0 / 15) and zero[0, 0] == 8          # (xmin, xmax) = (-1, +1)
+
+
+def test_all_non_negative_row_keeps_xmin_zero():
+    # quant.py:74-76 mirrors the range only when the row has a negative entry
+    row = np.array([[0.0, 0.25, 0.5, 1.0]], dtype=np.float32)
+    scale, zero = o.find_params_sym(row, 4)
+    assert scale[0, 0] == np.float32(1.0 / 15) and zero[0, 0] == 8
+    # the top of the range clips: 1.0/scale = 15 -> +8 -> clamp 15 -> dequant 7*scale
+    assert o.quantize_codes(row, scale, zero, 15)[0, 3] == 15
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_quantize_idempotent_and_bounded(bits):
+    rng = np.random.default_rng(1)
+    w = (rng.standard_normal((16, 64)) * 2e-3).astype(np.float32)
+    scale, zero = o.find_params_sym(w, bits)
+    maxq = 2 ** bits - 1
+    q1 = o.quantize(w, scale, zero, maxq)
+    q2 = o.quantize(q1, scale, zero, maxq)
+    assert np.array_equal(q1, q2)
+    lo, hi = -zero * scale, (maxq - zero) * scale
+    inside = (w >= lo) & (w <= hi)
+    assert np.all(np.abs(q1 - w)[inside] <= scale.repeat(64, 1)[inside] * 0.5000001)
+
+
+def test_group_scales_equal_per_group_rows():
+    rng = np.random.default_rng(2)
+    w = (rng.standard_normal((4, 256)) * 1e-3).astype(np.float32)
+    sg, zg = o.find_params_sym(w, 4, 128)
+    for g in range(2):
+        s1, _ = o.find_params_sym(w[:, 128 * g:128 * (g + 1)], 4)
+        assert np.array_equal(sg[:, g], s1[:, 0])
+
+
+def test_mask_brute_force_and_ties():
+    # every ordering of 4 distinct magnitudes: keep the two largest
+    for perm in itertools.permutations([1.0, 2.0, 3.0, 4.0]):
+        for signs in itertools.product([1, -1], repeat=4):
+            row = np.array([[p * s for p, s in zip(perm, signs)]], dtype=np.float32)
+            keep = o.prune_2of4_magnitude(row)[0]
+            assert sorted(np.abs(row[0])[keep].tolist()) == [3.0, 4.0]
+    # ties keep the lower index
+    assert o.prune_2of4_magnitude(np.array([[1, 1, 1, 1]], np.float32))[0].tolist() == [True, True, False, False]
+    assert o.prune_2of4_magnitude(np.array([[0, 0, 0, 5]], np.float32))[0].tolist() == [True, False, False, True]
+    assert o.prune_2of4_magnitude(np.array([[2, -3, 3, 2]], np.float32))[0].tolist() == [False, True, True, False]
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_compressed_delta_is_2of4(bits):
+    rng = np.random.default_rng(4)
+    d = (rng.standard_normal((32, 256)) * 1e-3).astype(np.float32)
+    codes, scales16, zeros, keep = o.compress_delta(d, bits)
+    zp = 2 ** (bits - 1)
+    assert np.all(zeros == zp)
+    c = codes.T.reshape(32, 64, 4)
+    assert np.all((c == zp).sum(axis=2) >= 2)          # at least two zero-point codes per group
+    assert np.all(keep.reshape(32, 64, 4).sum(axis=2) == 2)
+    assert np.all(codes.T[~keep] == zp)                # pruned entries carry the zero-point
