@@ -26,6 +26,7 @@ SIGNATURES = {
     "dz_multi_delta_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _sz, _vp]),
     "dz_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "dz_gemm_f16_pair": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_set_ksplit": (None, [_i]),
 }
 

@@ -17,8 +17,11 @@ namespace {
 constexpr int TM = 128, TN = 128, TK = 64;
 constexpr int LDS_STRIDE = TK + 8;  // halves; the pad keeps 16-byte row reads off shared banks
 
+// With w2 != nullptr the contraction runs over both weights, y = x @ w^T + x @ w2^T, in the same
+// fp32 accumulators (base weight and a dequantised delta, never summed in fp16).
 __global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict__ x,
                                                       const _Float16* __restrict__ w,
+                                                      const _Float16* __restrict__ w2,
                                                       _Float16* __restrict__ y, int T, int K, int N,
                                                       int accumulate, int ldy) {
   __shared__ __attribute__((aligned(16))) _Float16 sa[TM * LDS_STRIDE];
@@ -45,6 +48,9 @@ __global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict
       for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
 
   const int li = lane & 31, lh = lane >> 5;
+  const int npass = w2 ? 2 : 1;
+  for (int pass = 0; pass < npass; ++pass) {
+  const _Float16* wp = pass ? w2 : w;
   for (int k0 = 0; k0 < K; k0 += TK) {
     // stage: 128 rows x 64 halves per operand = 1024 chunks of 16 bytes, 4 per thread
 #pragma unroll
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict
       h8_t va = {0, 0, 0, 0, 0, 0, 0, 0};
       if (m0 + row < T) va = *(const h8_t*)(x + (size_t)(m0 + row) * K + k0 + ch * 8);
       *(h8_t*)(sa + row * LDS_STRIDE + ch * 8) = va;
-      const h8_t vb = *(const h8_t*)(w + (size_t)(n0 + row) * K + k0 + ch * 8);
+      const h8_t vb = *(const h8_t*)(wp + (size_t)(n0 + row) * K + k0 + ch * 8);
       *(h8_t*)(sb + row * LDS_STRIDE + ch * 8) = vb;
     }
     __syncthreads();
@@ -75,6 +81,7 @@ __global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict
           acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[b], fa[a], acc[a][b], 0, 0, 0);
     }
     __syncthreads();
+  }
   }
 #pragma unroll
   for (int a = 0; a < 2; ++a) {
@@ -102,14 +109,26 @@ __global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict
 
 }  // namespace
 
-extern "C" int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
-                           int accumulate, int ldy, void* stream) {
+static int gemm_launch(const uint16_t* x, const uint16_t* w, const uint16_t* w2, uint16_t* y, int T,
+                       int K, int N, int accumulate, int ldy, void* stream) {
   if (!x || !w || !y) return DZ_EINVAL;
   if (T < 1 || K < 1 || N < 1 || K % TK || N % TN || ldy < N || ldy % 4) return DZ_ESHAPE;
-  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)y & 7)) return DZ_EALIGN;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)w2 & 15) || ((uintptr_t)y & 7)) return DZ_EALIGN;
   const int total = ((T + TM - 1) / TM) * (N / TN);
   const int grid = (total + 7) / 8 * 8;
   hipLaunchKernelGGL(dz_gemm_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
-                     (const _Float16*)x, (const _Float16*)w, (_Float16*)y, T, K, N, accumulate, ldy);
+                     (const _Float16*)x, (const _Float16*)w, (const _Float16*)w2, (_Float16*)y, T, K, N,
+                     accumulate, ldy);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+extern "C" int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
+                           int accumulate, int ldy, void* stream) {
+  return gemm_launch(x, w, nullptr, y, T, K, N, accumulate, ldy, stream);
+}
+
+extern "C" int dz_gemm_f16_pair(const uint16_t* x, const uint16_t* w_a, const uint16_t* w_b, uint16_t* y,
+                                int T, int K, int N, int accumulate, int ldy, void* stream) {
+  if (!w_b) return DZ_EINVAL;
+  return gemm_launch(x, w_a, w_b, y, T, K, N, accumulate, ldy, stream);
 }

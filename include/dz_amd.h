@@ -89,8 +89,8 @@ size_t dz_workspace_bytes(int T, int K, int N);
  * indices [T] int64, -1 = base only, read on the device at execution time; y [T, ldy] fp16,
  * columns 0..N-1 written.  accumulate = 0: y = result; 1: y += result (fp32 add, one rounding).
  * Stands in for sbmm_4bit_2_4_native / ibmm_sparse_marlin at the call sites listed above.
- * T <= DZ_MAX_TOKENS_FUSED uses the single fused kernel; larger T runs the segment-wise
- * merge + matrix-core GEMM path and needs prefill workspace (dz_workspace_bytes covers it). */
+ * Requires 1 <= T <= DZ_MAX_TOKENS_FUSED (one fused launch).  Larger batches are served by the
+ * host wrapper from dz_segment + dz_dequant + dz_gemm_f16_pair, one GEMM per delta segment. */
 int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
                           const void* codes_stacked, const void* meta_stacked,
                           const void* scales_stacked, const int64_t* indices, uint16_t* y,
@@ -103,6 +103,13 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
  * (serving/vllm/model_executor/layers/linear.py:85-96) at prefill sizes. */
 int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
                 int accumulate, int ldy, void* stream);
+
+/* As dz_gemm_f16 with two weights of the same shape: y (+)= x @ w_a^T + x @ w_b^T, both products in
+ * the same fp32 accumulators.  Used at prefill sizes with w_a = base weight and w_b = one
+ * dequantised delta, so that base and delta are never added in fp16 (the reference's CPU path adds
+ * them in fp32: deltazip/utils/generate.py:9-20 as restated by the oracle). */
+int dz_gemm_f16_pair(const uint16_t* x, const uint16_t* w_a, const uint16_t* w_b, uint16_t* y,
+                     int T, int K, int N, int accumulate, int ldy, void* stream);
 
 /* Tuning hook used by the benchmark: override the split of K across workgroups of the fused
  * kernel (0 = automatic). */

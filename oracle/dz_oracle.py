@@ -202,7 +202,8 @@ def dequant_gptq(qweight, qzeros, scales16, g_idx, bits) -> np.ndarray:
     gi = g_idx.astype(np.int64)
     m = (codes.astype(np.int32) - zeros[gi].astype(np.int32)).astype(np.float32)
     s = scales16.astype(np.float16)[gi].astype(np.float32)
-    return (s * m).astype(np.float16)
+    with np.errstate(over="ignore"):       # products beyond the fp16 range round to inf, as in torch
+        return (s * m).astype(np.float16)
 
 
 # --------------------------------------------------------------------------------------

@@ -1,0 +1,87 @@
+"""GPU tests of the reference-shaped Python API: QuantLinear and the delta layers."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dz_oracle as o
+from deltazip_amd import (DeltaConfig, MergedColumnParallelLinearWithDelta, QuantLinear,
+                          RowParallelLinearWithDelta, convert_mapping, from_layer, ops)
+from _util import TOL, make_problem
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("bits,gs", [(4, -1), (2, -1), (4, 128)])
+def test_quant_linear_from_tensors_forward(dev, bits, gs):
+    """QuantLinear.from_tensors(...).forward(x) == x @ dequant(W) (quant_linear_naive.py:35-96)."""
+    dl = o.make_delta(64, 512, 2e-3, bits, gs, 42)
+    t = lambda a: torch.from_numpy(a).to(dev)
+    ql = QuantLinear.from_tensors(bits, t(dl["qweight"]), t(dl["qzeros"]), t(dl["scales"]), t(dl["g_idx"]), None, None)
+    assert (ql.infeatures, ql.outfeatures) == (512, 64)
+    x = torch.from_numpy(o.make_x(6, 512, 1)).to(dev).reshape(2, 3, 512)
+    y = ql(x)
+    assert y.shape == (2, 3, 64) and y.dtype == torch.float16
+    dt = o.dequant_gptq(dl["qweight"], dl["qzeros"], dl["scales"], dl["g_idx"], bits)
+    ref = x.reshape(6, 512).float().cpu().numpy() @ dt.astype(np.float32)
+    assert o.rel_err(y.reshape(6, 64).cpu().numpy(), ref) <= TOL
+    # the bias is added to the fp16 result, as the reference does (quant_linear_naive.py:82)
+    bias = (torch.randn(64, device=dev) * 0.01).half()
+    qb = QuantLinear.from_tensors(bits, t(dl["qweight"]), t(dl["qzeros"]), t(dl["scales"]), t(dl["g_idx"]), bias, None)
+    assert torch.equal(qb(x), y + bias)
+    w = ql.unpack().cpu().numpy()
+    assert np.array_equal(w.view(np.uint16), np.ascontiguousarray(dt.T).view(np.uint16))
+
+
+def test_layer_protocol(dev):
+    """create_delta_weights -> set_delta -> set_mapping -> forward; reset_delta; buffer rewrite."""
+    n, k, t, bits = 128, 512, 10, 4
+    p = make_problem(n, k, bits, -1, 3, t, "uniform", 7, dev)
+    base = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.float16)
+    with torch.no_grad():
+        base.weight.copy_(p["wb"])
+    cfg = DeltaConfig(max_deltas=4, max_bitwidth=bits)
+    layer = from_layer(base, 4, cfg, ["gate_proj", "up_proj"])
+    assert isinstance(layer, MergedColumnParallelLinearWithDelta)
+    assert tuple(layer.qweight_stacked.shape) == (4, k // 32, 2 * n)
+    assert tuple(layer.meta_stacked.shape) == (4, n, k // 16) and tuple(layer.scales_stacked.shape) == (4, 1, n)
+    # slots 1..3 take the deltas: native tensors for two, GPTQ tensors (converted on the fly) for one
+    layer.set_delta(1, bits, p["q"][0].cpu().pin_memory(), None, p["s"][0].cpu().pin_memory(), None, p["m"][0].cpu().pin_memory())
+    layer.set_delta(2, bits, p["q"][1], None, p["s"][1], None, p["m"][1])
+    g = p["gptq"][2]
+    layer.set_delta(3, bits, torch.from_numpy(g["qweight"]), torch.from_numpy(g["qzeros"]),
+                    torch.from_numpy(g["scales"]), torch.from_numpy(g["g_idx"]), None)
+    assert layer.bitwidth == [0, bits, bits, bits]
+    # manager side: delta ids 11, 12, 13 live in slots 1, 2, 3; id 0 = base
+    index_buf = torch.full((16,), -1, dtype=torch.int64, device=dev)
+    slot_ids = [None, 11, 12, 13]
+    token_ids = [11, 0, 13, 12, 12, 0, 11, 13, 13, 11]
+    idx = convert_mapping(token_ids, slot_ids, out=index_buf)
+    layer.set_mapping(index_buf, None, None, None, [t])
+    out, out_bias = layer(p["x"])
+    assert out_bias is None
+    oracle_ids = np.array([{0: -1, 11: 0, 12: 1, 13: 2}[i] for i in token_ids])
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], oracle_ids)
+    assert o.rel_err(out.cpu().numpy(), ref) <= TOL
+    # reset a slot: its tokens fall back to the base layer
+    layer.reset_delta(2)
+    out2, _ = layer(p["x"])
+    ids2 = np.where(oracle_ids == 1, -1, oracle_ids)
+    assert o.rel_err(out2.cpu().numpy(), o.forward_ref(p["x_np"], p["wb_np"], p["dts"], ids2)) <= TOL
+    # the mapping buffer is rewritten in place for the next step
+    convert_mapping([13] * t, slot_ids, out=index_buf)
+    out3, _ = layer(p["x"])
+    assert o.rel_err(out3.cpu().numpy(), o.forward_ref(p["x_np"], p["wb_np"], p["dts"], np.full(t, 2))) <= TOL
+    with pytest.raises(ValueError):
+        layer.set_delta(0, 2, p["q"][0], None, p["s"][0], None, p["m"][0])      # wrong bit width
+
+
+def test_row_parallel_rejects_bias_and_from_layer_passthrough(dev):
+    lin = torch.nn.Linear(512, 64, bias=True, device=dev, dtype=torch.float16)
+    cfg = DeltaConfig(max_deltas=1, max_bitwidth=4)
+    layer = from_layer(lin, 1, cfg, [])
+    assert isinstance(layer, RowParallelLinearWithDelta)
+    layer.set_mapping(torch.full((4,), -1, dtype=torch.int64, device=dev), indices_len=[4])
+    with pytest.raises(ValueError, match="bias"):
+        layer(torch.zeros(4, 512, dtype=torch.float16, device=dev))
+    act = torch.nn.ReLU()
+    assert from_layer(act, 1, cfg, []) is act

@@ -1,0 +1,224 @@
+"""GPU parity tests: every entry point is called through the C ABI (via the ctypes wrapper) and
+compared with the CPU oracle on the same seeded inputs.  Dequantised deltas must match bit for
+bit; layer outputs within TOL = 1e-2 max relative error (fp16 outputs vs the fp32 reference)."""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dz_oracle as o
+from deltazip_amd import ops
+from _util import TOL, make_problem, run_layer
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("gs", [-1, 64, 128, 256])
+def test_dequant_bit_exact(dev, bits, gs):
+    p = make_problem(96, 768, bits, gs, 2, 1, "single", 100 + bits + max(gs, 0), dev)
+    for d in range(2):
+        got = ops.dequant(p["q"][d], p["m"][d], p["s"][d], 768, 96, bits).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(p["dts"][d].T).view(np.uint16))
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_dequant_extreme_scales(dev, bits):
+    """Subnormal, tiny and huge fp16 scales: one rounding of the exact product, no flush to zero."""
+    k, n = 256, 32
+    zp = 2 ** (bits - 1)
+    rng = np.random.default_rng(5)
+    codes = np.full((k, n), zp, dtype=np.uint8)
+    pos = rng.integers(0, 4, size=(k // 4, n))
+    for g in range(k // 4):                       # one non-zero code per group of 4
+        codes[4 * g + pos[g], np.arange(n)] = rng.integers(0, 2 ** bits, size=n)
+    scales = np.array([6e-8, 1.2e-7, 3e-6, 6.1e-5, 1e-3, 0.5, 1000.0, 8000.0] * 4, dtype=np.float16).reshape(1, n)
+    qw, qz, sc, gi = o.pack_codes_gptq(codes, np.full((1, n), zp), scales, bits)
+    ref = o.dequant_gptq(qw, qz, sc, gi, bits)
+    q, m, s = ops.repack_gptq_to_native(torch.from_numpy(qw), torch.from_numpy(qz), torch.from_numpy(sc),
+                                        torch.from_numpy(gi), bits)
+    got = ops.dequant(q.to(dev), m.to(dev), s.to(dev), k, n, bits).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(ref.T).view(np.uint16))
+    assert np.any((ref != 0) & (np.abs(ref.astype(np.float32)) < 6.1e-5))   # subnormals were exercised
+
+
+def test_merge_is_fp32_add_rounded_once(dev):
+    p = make_problem(64, 512, 4, -1, 1, 1, "single", 31, dev)
+    got = ops.merge(p["wb"], p["q"][0], p["m"][0], p["s"][0], 4).cpu().numpy()
+    ref = (p["wb_np"].astype(np.float32) + p["dts"][0].T.astype(np.float32)).astype(np.float16)
+    assert np.array_equal(got.view(np.uint16), ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("t,s", [(1, 1), (9, 8), (128, 5), (1000, 3), (4099, 17)])
+def test_segment(dev, t, s):
+    rng = np.random.default_rng(t)
+    ids = rng.integers(-1, s, size=t).astype(np.int64)
+    ids[::7] = s + 3                               # out-of-range ids count as -1
+    perm, off = ops.segment(torch.from_numpy(ids).to(dev), s)
+    key = np.where((ids < 0) | (ids >= s), -1, ids)
+    assert np.array_equal(perm.cpu().numpy(), np.argsort(key, kind="stable"))
+    counts = [(key == v).sum() for v in range(-1, s)]
+    assert off.cpu().numpy().tolist() == [0] + np.cumsum(counts).tolist()
+
+
+CASES = [
+    # n, k, bits, gs, deltas, tokens, ids
+    (64, 512, 2, -1, 3, 5, "uniform"),
+    (64, 512, 4, -1, 3, 16, "uniform"),
+    (96, 768, 2, -1, 2, 1, "single"),
+    (96, 768, 4, 64, 2, 17, "uniform"),
+    (128, 1024, 2, 128, 4, 32, "uniform"),
+    (128, 1024, 4, 128, 4, 32, "zipf"),
+    (160, 1280, 2, -1, 8, 31, "uniform"),
+    (256, 1024, 2, -1, 6, 48, "uniform"),
+    (256, 1024, 4, -1, 6, 64, "zipf"),
+    (256, 2048, 2, 256, 5, 100, "uniform"),
+    (256, 1024, 4, 128, 12, 128, "zipf"),
+    (32, 256, 2, -1, 1, 33, "single"),
+]
+
+
+@pytest.mark.parametrize("n,k,bits,gs,nd,t,kind", CASES)
+def test_layer_parity(dev, n, k, bits, gs, nd, t, kind):
+    p = make_problem(n, k, bits, gs, nd, t, kind, 1000 + n + k + t, dev)
+    if t > 2:
+        p["ids_np"][1] = -1
+        p["ids"] = torch.from_numpy(p["ids_np"]).to(dev)
+    y = run_layer(p).cpu().numpy()
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    assert o.rel_err(y, ref) <= TOL
+    assert ops.workspace_status() == 0
+
+
+def test_edge_cases(dev):
+    p = make_problem(64, 512, 4, -1, 2, 12, "uniform", 77, dev)
+    base = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], np.full(12, -1))
+    # every token base-only == plain linear layer
+    p["ids"] = torch.full((12,), -1, dtype=torch.int64, device=dev)
+    assert o.rel_err(run_layer(p).cpu().numpy(), base) <= TOL
+    # no slots at all (S = 0 is not allowed by the stacked tensors; one reset slot stands in)
+    # a reset slot (zero scales) contributes exactly nothing
+    p["s"].zero_()
+    p["ids"] = torch.zeros(12, dtype=torch.int64, device=dev)
+    y0 = run_layer(p)
+    p["ids"] = torch.full((12,), -1, dtype=torch.int64, device=dev)
+    assert torch.equal(y0, run_layer(p))
+
+
+def test_out_of_range_ids_are_flagged_and_treated_as_base(dev):
+    p = make_problem(64, 512, 2, -1, 2, 8, "uniform", 78, dev)
+    ids = p["ids_np"].copy(); ids[3] = 2; ids[5] = -7
+    p["ids"] = torch.from_numpy(ids).to(dev)
+    y = run_layer(p).cpu().numpy()
+    assert ops.workspace_status() & 1
+    ids_eff = np.where((ids < 0) | (ids >= 2), -1, ids)
+    assert o.rel_err(y, o.forward_ref(p["x_np"], p["wb_np"], p["dts"], ids_eff)) <= TOL
+    ops._workspaces.clear()                        # fresh (zeroed) status word for later tests
+
+
+GOLDEN = sorted(glob.glob(os.path.join(os.path.dirname(__file__), "golden", "*.npz")))
+
+
+@pytest.mark.parametrize("path", GOLDEN, ids=[os.path.basename(p)[:-4] for p in GOLDEN])
+def test_golden_fixtures(dev, path):
+    g = np.load(path)
+    bits = int(g["bits"])
+    nd = sum(1 for k in g.files if k.endswith("_qweight"))
+    qs, ms, ss = [], [], []
+    for d in range(nd):
+        q, m, s = ops.repack_gptq_to_native(*(torch.from_numpy(g[f"d{d}_{k}"]) for k in
+                                              ("qweight", "qzeros", "scales", "g_idx")), bits)
+        K, N = g[f"d{d}_dequant_t"].shape
+        got = ops.dequant(q.to(dev), m.to(dev), s.to(dev), K, N, bits).cpu().numpy()
+        assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(g[f"d{d}_dequant_t"].T).view(np.uint16))
+        qs.append(q); ms.append(m); ss.append(s)
+    q, m, s = (torch.stack(v).to(dev) for v in (qs, ms, ss))
+    x = torch.from_numpy(g["x"]).to(dev); ids = torch.from_numpy(g["ids"]).to(dev)
+    y = ops.apply_delta(x, q, s, m, ids, torch.from_numpy(g["w_base"]).to(dev)).cpu().numpy()
+    assert o.rel_err(y, g["y_ref"]) <= TOL
+    yd = torch.zeros_like(torch.from_numpy(g["y_delta_only"])).half().to(dev)
+    ops.add_delta(yd, x, q, None, s, None, ids, meta=m)
+    assert o.rel_err(yd.cpu().numpy(), g["y_delta_only"]) <= TOL
+
+
+def test_add_delta_slices_qkv_and_gate_up(dev):
+    """In-place y[:, off:off+n] += x @ delta^T per output slice (deltazip.py:40-153)."""
+    k, t = 512, 20
+    slices = (128, 64, 64)                         # q, k, v
+    probs = [make_problem(n, k, 4, -1, 3, t, "uniform", 300 + i, dev) for i, n in enumerate(slices)]
+    ids_np = probs[0]["ids_np"]; ids = probs[0]["ids"]; x = probs[0]["x"]; x_np = probs[0]["x_np"]
+    y0 = (torch.randn(t, sum(slices), device=dev) * 0.05).half()
+    y = y0.clone()
+    off = 0
+    for p, n in zip(probs, slices):
+        ops.add_delta_slice(y, x, p["q"], None, p["s"], None, ids, 1.0, off, n, meta=p["m"])
+        off += n
+    torch.cuda.synchronize()
+    off = 0
+    for p, n in zip(probs, slices):
+        ref = y0[:, off:off + n].float().cpu().numpy() + o.forward_ref(x_np, None, p["dts"], ids_np)
+        assert o.rel_err(y[:, off:off + n].cpu().numpy(), ref) <= TOL
+        off += n
+    # whole-width form
+    p = probs[0]
+    yy = torch.zeros(t, 128, dtype=torch.float16, device=dev)
+    assert ops.add_delta(yy, x, p["q"], None, p["s"], None, ids, meta=p["m"]) is yy
+    assert o.rel_err(yy.cpu().numpy(), o.forward_ref(x_np, None, p["dts"], ids_np)) <= TOL
+
+
+def test_deterministic_and_order_independent(dev):
+    p = make_problem(128, 1024, 2, -1, 5, 32, "uniform", 55, dev)
+    y1 = run_layer(p); y2 = run_layer(p)
+    assert torch.equal(y1, y2)                     # run-to-run bit identical (no float atomics)
+    perm = torch.randperm(32, device=dev)
+    q = dict(p); q["x"] = p["x"][perm].contiguous(); q["ids"] = p["ids"][perm].contiguous()
+    assert torch.equal(run_layer(q), y1[perm])     # a token's result does not depend on its position
+    srt = torch.argsort(p["ids"], stable=True)
+    q["x"] = p["x"][srt].contiguous(); q["ids"] = p["ids"][srt].contiguous()
+    assert torch.equal(run_layer(q), y1[srt])
+
+
+@pytest.mark.parametrize("t", [32, 100])
+def test_k_split_variants_agree(dev, t):
+    p = make_problem(64, 2048, 4, 128, 3, t, "uniform", 66, dev)
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    try:
+        for ns in (1, 2, 3, 8):
+            ops.set_ksplit(ns)
+            assert o.rel_err(run_layer(p).cpu().numpy(), ref) <= TOL
+            assert torch.equal(run_layer(p), run_layer(p))
+    finally:
+        ops.set_ksplit(0)
+
+
+def test_indices_are_read_at_call_time(dev):
+    """The manager rewrites the index buffer between steps (models.py:421-430); the layer must see it."""
+    p = make_problem(64, 512, 4, -1, 3, 8, "uniform", 88, dev)
+    buf = torch.zeros(16, dtype=torch.int64, device=dev)
+    view = buf[:8]
+    for ids in ([0, 1, 2, -1, 0, 1, 2, -1], [2, 2, 2, 2, -1, -1, 0, 0]):
+        buf[:8].copy_(torch.tensor(ids))
+        y = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], view, p["wb"]).cpu().numpy()
+        assert o.rel_err(y, o.forward_ref(p["x_np"], p["wb_np"], p["dts"], np.array(ids))) <= TOL
+
+
+def test_gemm_f16(dev):
+    from deltazip_amd.prefill import gemm_f16
+    torch.manual_seed(0)
+    x = torch.randn(300, 512, device=dev).half(); w = (torch.randn(256, 512, device=dev) * 0.05).half()
+    y = gemm_f16(x, w)
+    ref = x.float() @ w.float().t()
+    assert o.rel_err(y.float().cpu().numpy(), ref.cpu().numpy()) <= 2e-3
+    y2 = y.clone(); gemm_f16(x, w, y2, accumulate=True)
+    assert o.rel_err(y2.float().cpu().numpy(), 2 * ref.cpu().numpy()) <= 3e-3
+
+
+@pytest.mark.parametrize("kind", ["blocks", "uniform"])
+def test_prefill_sized_call(dev, kind):
+    """T > 128: per-segment merge + matrix-core GEMM; sorted (one delta per request) and unsorted."""
+    p = make_problem(256, 1024, 2, -1, 4, 400, kind, 99, dev)
+    y = run_layer(p).cpu().numpy()
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    assert o.rel_err(y, ref) <= TOL
