@@ -39,9 +39,16 @@ __device__ __forceinline__ uint32_t pkfma(uint32_t v, float mul, float add) {
   return r.u;
 }
 
+// v_and_or_b32 takes one scalar operand at most: the masks live in scalar registers, the magic
+// constant in a vector register (the asm keeps the compiler from turning it back into a literal).
+__device__ __forceinline__ uint32_t magic_vgpr() {
+  uint32_t m = 0x64006400u;
+  asm volatile("" : "+v"(m));
+  return m;
+}
+
 // 2-bit: one word holds both fragments (s = 0, 1) of a step.
-__device__ __forceinline__ void unpack2(uint32_t w, h8_t& a0, h8_t& a1) {
-  const uint32_t MAGIC = 0x64006400u;
+__device__ __forceinline__ void unpack2(uint32_t w, uint32_t MAGIC, h8_t& a0, h8_t& a1) {
   const uint32_t w2 = w >> 10;
   H8U r0, r1;
   r0.u[0] = pkfma((w & 0x00030003u) | MAGIC, 1.0f, -1026.0f);
@@ -57,8 +64,7 @@ __device__ __forceinline__ void unpack2(uint32_t w, h8_t& a0, h8_t& a1) {
 }
 
 // 4-bit: one word holds one fragment.
-__device__ __forceinline__ h8_t unpack4(uint32_t w) {
-  const uint32_t MAGIC = 0x64006400u;
+__device__ __forceinline__ h8_t unpack4(uint32_t w, uint32_t MAGIC) {
   const uint32_t w2 = w >> 8;
   H8U r;
   r.u[0] = pkfma((w & 0x000F000Fu) | MAGIC, 1.0f, -1032.0f);
@@ -67,7 +73,6 @@ __device__ __forceinline__ h8_t unpack4(uint32_t w) {
   r.u[3] = pkfma((w2 & 0x00F000F0u) | MAGIC, 0.0625f, -72.0f);
   return r.h;
 }
-
 
 struct MdlParams {
   const _Float16* x;

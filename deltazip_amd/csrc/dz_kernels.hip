@@ -160,6 +160,7 @@ __global__ __launch_bounds__(64 * WN * WK) void dz_mdl_kernel(const MdlParams P)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wn = wave % WN, wk = wave / WN;
   const int jj = lane & 15, ga = lane >> 4;
+  const uint32_t MAGIC = magic_vgpr();
 
   // workgroup -> (n-pair group, k-chunk); the chunks of one n-pair group sit on one XCD
   // (workgroups are dealt round-robin over the 8 XCDs) so their partial sums meet in one L2
@@ -320,10 +321,10 @@ __global__ __launch_bounds__(64 * WN * WK) void dz_mdl_kernel(const MdlParams P)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
               if (BITS == 2) {
-                unpack2(cur.code[0][j], A[j][0], A[j][1]);
+                unpack2(cur.code[0][j], MAGIC, A[j][0], A[j][1]);
               } else {
-                A[j][0] = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 0]);
-                A[j][1] = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 1]);
+                A[j][0] = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 0], MAGIC);
+                A[j][1] = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 1], MAGIC);
               }
             }
             if (PRE) {

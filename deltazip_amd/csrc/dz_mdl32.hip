@@ -3,18 +3,17 @@
 // One workgroup = 4 wavefronts = one n-pair (32 output rows) x a chunk of k-blocks; each
 // wavefront owns whole k-blocks (256 input columns) of that n-pair and is self-sufficient until
 // the final reduction:
-//   * at entry it issues, back to back, the loads of its activations slice (straight into LDS,
-//     global_load_lds_dwordx4), of the token ids and of its 32 x 256 base-weight tile (16 x
-//     128-bit loads per lane), so HBM traffic starts at once;
-//   * the token ids arrive through scalar loads (a path that does not queue behind the vector
-//     loads); the distinct deltas of the batch are enumerated with ballots (no sort, no barrier):
-//     output columns stay in token order and each delta gets a per-column mask.  Batches that
-//     arrive sorted by id (as the reference's scheduler delivers them) touch fewer column tiles;
-//   * the packed words of the first deltas are then requested together;
-//   * base tile x activations runs on v_mfma_f32_16x16x32_f16, each delta on the 2:4-sparse
-//     v_smfmac_f32_16x16x64_f16 with the unpacked codes as the sparse operand and the stored
-//     positions as its index operand; the dense operand (activations) is read from the
-//     wavefront's own LDS slice;
+//   * at entry it requests its activations slice (straight into LDS, global_load_lds_dwordx4) and
+//     its 32 x 256 base-weight tile (16 x 128-bit loads per lane), so HBM traffic starts at once;
+//   * the token ids are fetched first; the distinct deltas of the batch are enumerated
+//     with ballots (no sort, no barrier): output columns stay in token order and each delta gets a
+//     per-column mask.  Batches that arrive sorted by id (as the reference's scheduler delivers
+//     them) touch fewer column tiles;
+//   * the packed words of up to 8 deltas (two batches of 4) are then requested together;
+//   * compute runs column tile by column tile: one read of the dense operand (activations, from
+//     the wavefront's own LDS slice) feeds the base product (v_mfma_f32_16x16x32_f16) and the
+//     products of every delta of the current batch (2:4-sparse v_smfmac_f32_16x16x64_f16, unpacked
+//     codes as the sparse operand, stored positions as its index operand);
 //   * partial sums of the 4 wavefronts meet in LDS; when K is split over several workgroups the
 //     per-chunk sums go to a workspace and the last workgroup to arrive adds them in a fixed
 //     order (deterministic) and writes y.
@@ -27,16 +26,17 @@ constexpr int WK32 = 4;
 
 template <int BITS, int TT, bool PRE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
-  constexpr int TP = 16 * TT;                  // padded token count (16 or 32)
-  constexpr int PD = (BITS == 2) ? (TT == 1 ? 8 : 6) : 4;  // deltas in flight per wavefront
-  constexpr int NX = TP / 2;                   // activation loads per wavefront (2 rows each)
+  constexpr int TP = 16 * TT;              // padded token count (16 or 32)
+  constexpr int G = (BITS == 2) ? 4 : (TT == 2 ? 2 : 3);   // deltas per batch; two batches are in flight
+  constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform, in a scalar register
   const int jj = lane & 15, ga = lane >> 4;
+  const uint32_t MAGIC = magic_vgpr();
   _Float16* xw = (_Float16*)smem + (size_t)wave * TP * DZ_KBLOCK;   // this wavefront's activations
-  f4_t* red = (f4_t*)smem;                                   // reduction buffer, after the barrier
+  f4_t* red = (f4_t*)smem;                                          // reduction buffer, after the barrier
 
   // workgroup -> (n-pair, k-chunk); the chunks of one n-pair are dealt to one XCD so that their
   // partial sums can meet in that XCD's L2
@@ -46,27 +46,8 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   const int n0 = np * DZ_NPAIR;
   const int kb_lo = kc * P.cb, kb_hi = min(P.NKB, kb_lo + P.cb);
   const int nrounds = (kb_hi - kb_lo + WK32 - 1) / WK32;
+  const unsigned Kb = (unsigned)P.K * 2u;  // row pitch of x and w_base in bytes
   DZ_TS(0);
-  // token ids first, through scalar loads (wavefront-uniform addresses): lane t keeps the key of
-  // token t.  key: 0 = base only, id + 1 otherwise, INT_MAX for padding lanes.
-  int key = 0x7fffffff;
-  {
-    long long ids[TP];
-#pragma unroll
-    for (int t = 0; t < TP; ++t) ids[t] = P.idx[min(t, P.T - 1)];
-    bool bad = false;
-#pragma unroll
-    for (int t = 0; t < TP; ++t) {
-      const long long v = ids[t];
-      const int k = (v < 0 || v >= P.S) ? 0 : (int)v + 1;
-      bad |= (v < -1 || v >= P.S);
-      if (t < P.T) key = (lane == t) ? k : key;
-    }
-    if (bad && blockIdx.x == 0 && tid == 0) atomicOr(P.status, 1u);
-  }
-  // tokens that carry a delta; lanes >= T never match
-  const unsigned long long mdelta = __builtin_amdgcn_ballot_w64(key != 0 && key != 0x7fffffff);
-  DZ_TS(1);
 
   f4_t accb[2][TT], accd[2][TT];
 #pragma unroll
@@ -77,8 +58,9 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
       accd[s][tt] = (f4_t){0.f, 0.f, 0.f, 0.f};
     }
 
-  // LDS byte offsets of this lane's operand chunks: row = token tt*16 + jj, chunk index
-  // 8*j + 4*h + ga with its low 4 bits swizzled by the row; index = (j & 1) * 2 + h
+  // LDS byte offsets of this lane's operand chunks: row = token tt*16 + jj (512 bytes per row),
+  // chunk index 8*j + 4*h + ga with its low 4 bits XOR-swizzled by the row so that the 16 rows of
+  // one operand read fall on different banks; index = (j & 1) * 2 + h, (j >> 1) adds 256 bytes
   int boff[TT][4];
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt)
@@ -86,62 +68,25 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     for (int c = 0; c < 4; ++c)
       boff[tt][c] = (tt * 16 + jj) * (DZ_KBLOCK * 2) + ((((c << 2) | ga) ^ jj) << 4);
 
-  for (int r = 0; r < nrounds; ++r) {
-    const int kb = kb_lo + r * WK32 + wave;
-    const bool active = kb < kb_hi;  // wavefront-uniform
-    // Per-round copy of the lane id that the optimiser cannot prove loop-invariant: otherwise it
-    // precomputes every load offset of the round outside the loop and spills them.
-    int lane_r = lane;
-    asm volatile("" : "+v"(lane_r));
-    const int jj_r = lane_r & 15, ga_r = lane_r >> 4;
+  u4_t a[2][4][2];  // base tile: [row fragment][step][half]
 
-    // ---- issue order: [later rounds: packed deltas], activations slice (L2 -> LDS directly), base
-    // tile (HBM).  LDS row t = token t, 512 bytes, its 16-byte chunks XOR-swizzled with (t & 15)
-    // so that the 16 rows one operand read gathers fall on different banks.  Rows >= T repeat row
-    // T-1: they only feed output columns that are never stored.
-    // Addresses are a wavefront-uniform base plus one 32-bit lane offset.
-    u4_t a[2][4][2];
-    const unsigned Kb = (unsigned)P.K * 2u;  // row pitch in bytes
-    // ---- delta walk: pop the lowest token that still has an unvisited delta, take its id and
-    // clear every token of that delta (all scalar work)
-    unsigned long long m_use = mdelta, m_load = mdelta;
-    auto pop = [&](unsigned long long& m, int& d, unsigned long long& dm) {
-      const int l = __builtin_ctzll(m);
-      const int kd = __builtin_amdgcn_readlane(key, l);
-      dm = __builtin_amdgcn_ballot_w64(key == kd);
-      m &= ~dm;
-      d = kd - 1;
-    };
-    Frag<BITS> ring[PD];
-    auto fill_ring = [&]() {
+  // Activations slice of k-block kb -> LDS, rows in token order; rows >= T repeat row T-1 (they
+  // only feed output columns that are never stored).  Then the base tile.  Addresses are a
+  // wavefront-uniform base plus one 32-bit lane offset.
+  auto issue_x_and_base = [&](int kb, int lane_r) {
+    const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
 #pragma unroll
-      for (int u = 0; u < PD; ++u)
-        if (m_load) {
-          int d;
-          unsigned long long dm;
-          pop(m_load, d, dm);
-          ring[u] = load_frag<BITS>(P, d, np, kb, lane_r);
-        }
-    };
-    // the packed words of the first deltas go out first
-    if (active) fill_ring();
-    __builtin_amdgcn_sched_barrier(0);
-    if (active) {
-      const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
-#pragma unroll
-      for (int i = 0; i < NX; ++i) {
-        const int t = min(2 * i + (lane_r >> 5), P.T - 1), c = lane_r & 31;
-        const unsigned off = (unsigned)t * Kb + (unsigned)((c ^ (t & 15)) << 4);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
-                                         (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
-                                         16, 0, 0);
-      }
+    for (int i = 0; i < NX; ++i) {
+      const int t = min(2 * i + (lane_r >> 5), P.T - 1), c = lane_r & 31;
+      const unsigned off = (unsigned)t * Kb + (unsigned)((c ^ (t & 15)) << 4);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
+                                       (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
+                                       16, 0, 0);
     }
-
     __builtin_amdgcn_sched_barrier(0);
-    if (active && P.wb) {
+    if (P.wb) {
       const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
-      const unsigned loff = (unsigned)jj_r * Kb + (unsigned)ga_r * 16u;
+      const unsigned loff = (unsigned)(lane_r & 15) * Kb + (unsigned)(lane_r >> 4) * 16u;
 #pragma unroll
       for (int s = 0; s < 2; ++s) {
         const char* ws = wbb + (size_t)(16 * s) * Kb;
@@ -153,31 +98,118 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+  };
 
-    // Loads return in order: once at most the 16 base loads are outstanding, the packed deltas and
-    // this wavefront's LDS slice are complete.  (The compiler
-    // does not order LDS reads after LDS-direct loads by itself.)
+  // token ids: lane t keeps the key of token t (0 = base only, id + 1 otherwise, INT_MAX for
+  // padding lanes); mdelta marks the tokens that carry a delta.  Both are set in round 0.
+  int key = 0x7fffffff;
+  unsigned long long mdelta = 0;
+  // The ids are requested before anything else and nothing more is requested until they are in:
+  // a request queued behind this kernel's own flood of weight loads takes several microseconds.
+  long long id = -1;
+  if (lane < P.T) id = P.idx[lane];
+  __builtin_amdgcn_sched_barrier(0);
+
+  for (int r = 0; r < nrounds; ++r) {
+    const int kb = kb_lo + r * WK32 + wave;
+    const bool active = kb < kb_hi;  // wavefront-uniform
+    // Per-round copy of the lane id that the optimiser cannot prove loop-invariant: otherwise it
+    // precomputes every load offset of the round outside the loop and spills them.
+    int lane_r = lane;
+    asm volatile("" : "+v"(lane_r));
+
+    // ---- delta walk.  Visits are (column tile, delta) pairs: tiles in order, inside a tile the
+    // distinct deltas in order of first token.  They are cut into batches of at most G that never
+    // span tiles; every tile gets at least one (possibly empty) batch.  The loader runs two
+    // batches ahead of the consumer; both follow the same rule, with scalar state only.
+    Frag<BITS> ring[2][G];
+    int ld_tt = 0;
+    unsigned long long ld_m = mdelta & 0xffffull;
+    auto tile_bits = [&](int tt) -> unsigned long long { return (mdelta >> (16 * tt)) & 0xffffull; };
+    auto pop = [&](unsigned long long& m, int tt, int& kd, unsigned& cols) {
+      const int l = __builtin_ctzll(m) + 16 * tt;
+      kd = __builtin_amdgcn_readlane(key, l);
+      const unsigned long long dm = (__builtin_amdgcn_ballot_w64(key == kd) >> (16 * tt)) & 0xffffull;
+      m &= ~dm;
+      cols = (unsigned)dm;  // columns of this tile that belong to the delta
+    };
+    auto load_batch = [&](Frag<BITS> (&slot)[G]) {
+      if (ld_tt >= TT) return;
+#pragma unroll
+      for (int g = 0; g < G; ++g)
+        if (ld_m) {
+          int kd;
+          unsigned cols;
+          pop(ld_m, ld_tt, kd, cols);
+          slot[g] = load_frag<BITS>(P, kd - 1, np, kb, lane_r);
+        }
+      if (ld_m == 0) {
+        ++ld_tt;
+        if (ld_tt < TT) ld_m = tile_bits(ld_tt);
+      }
+    };
+
+    // Issue order: packed deltas, activations, base tile.  In round 0 nothing is requested before
+    // the ids are in: a request queued behind this kernel's own flood of weight loads would take
+    // far longer than the ids do on an idle memory system, and the packed deltas depend on them.
+    if (r == 0) {
+      if (lane < P.T) {
+        key = (id < 0 || id >= P.S) ? 0 : (int)id + 1;
+        if ((id < -1 || id >= P.S) && blockIdx.x == 0 && wave == 0) atomicOr(P.status, 1u);
+      }
+      // tokens that carry a delta; lanes >= T never match
+      mdelta = __builtin_amdgcn_ballot_w64(key != 0 && key != 0x7fffffff);
+      ld_m = mdelta & 0xffffull;
+      DZ_TS(1);
+    }
+    if (active) {
+      load_batch(ring[0]);
+      load_batch(ring[1]);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (active) issue_x_and_base(kb, lane_r);
+    __builtin_amdgcn_sched_barrier(0);
+    if (r == 0) DZ_TS(2);
+    // Loads return in order and the base tile (16 loads) was requested last: once at most 16 loads
+    // are outstanding, the packed deltas and this wavefront's LDS slice are complete.  (The
+    // compiler does not order LDS reads after LDS-direct loads by itself.)
     if (P.wb) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
+    if (r == 0) DZ_TS(3);
 
     if (active) {
-      if (r == 0) DZ_TS(2);
-
-      // chunk index of step j, half h is 8*j + 4*h + ga; its low 4 bits are swizzled per row
       auto ldsB = [&](int tt, int j, h8_t& lo, h8_t& hi) {
         const char* p = (const char*)xw + (j >> 1) * 256;
         lo = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 0]);
         hi = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 1]);
       };
-      // ---- base: dense matrix-core product over all token tiles
-      if (P.wb) {
+      // one batch of one column tile: every operand read feeds the base product (first batch of
+      // the tile only) and all deltas of the batch
+      auto consume = [&](int tt, Frag<BITS> (&slot)[G], unsigned long long& m, bool with_base) {
+        int kd[G];
+        unsigned cols[G];
+        int nb = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int g = 0; g < G; ++g) {
+          kd[g] = 0;
+          cols[g] = 0;
+          if (m) {
+            pop(m, tt, kd[g], cols[g]);
+            nb = g + 1;
+          }
+        }
+        f4_t t0[G], t1[G];
 #pragma unroll
-          for (int tt = 0; tt < TT; ++tt) {
-            h8_t blo, bhi;
-            ldsB(tt, j, blo, bhi);
+        for (int g = 0; g < G; ++g) {
+          t0[g] = (f4_t){0.f, 0.f, 0.f, 0.f};
+          t1[g] = (f4_t){0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h8_t blo, bhi;
+          ldsB(tt, j, blo, bhi);
+          if (with_base && P.wb) {
 #pragma unroll
             for (int s = 0; s < 2; ++s) {
               H8U a0, a1;
@@ -187,78 +219,64 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
               accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1.h, bhi, accb[s][tt], 0, 0, 0);
             }
           }
-      }
-      if (r == 0) DZ_TS(4);
-
-      // ---- deltas: sparse matrix-core product, one delta at a time
-      while (m_use) {
+          const h16_t B = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12,
+                                                  13, 14, 15);
 #pragma unroll
-        for (int u = 0; u < PD; ++u) {
-          if (m_use) {
-            int d;
-            unsigned long long dm;
-            pop(m_use, d, dm);
-            const Frag<BITS> cur = ring[u];
-            if (m_load) {
-              int d2;
-              unsigned long long dm2;
-              pop(m_load, d2, dm2);
-              ring[u] = load_frag<BITS>(P, d2, np, kb, lane_r);
-            }
-            // lane's operand row is n0 + 16*s + jj; one scale per (row, K-group) when PRE
-            const _Float16* sp = P.scales + (size_t)d * P.scales_slot + n0 + jj;
-            _Float16 s0 = (_Float16)0.f, s1 = (_Float16)0.f;
-            int gprev = -1;
-            f4_t t0[TT], t1[TT];
-            bool in[TT];
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt) {
-              t0[tt] = (f4_t){0.f, 0.f, 0.f, 0.f};
-              t1[tt] = (f4_t){0.f, 0.f, 0.f, 0.f};
-              in[tt] = (dm >> (tt * 16 + jj)) & 1ull;
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
+          for (int g = 0; g < G; ++g) {
+            if (g < nb) {
               h8_t A0, A1;
               if (BITS == 2) {
-                unpack2(cur.code[0][j], A0, A1);
+                unpack2(slot[g].code[0][j], MAGIC, A0, A1);
               } else {
-                A0 = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 0]);
-                A1 = unpack4(cur.code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 1]);
+                A0 = unpack4(slot[g].code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 0], MAGIC);
+                A1 = unpack4(slot[g].code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 1], MAGIC);
               }
               if (PRE) {
-                const int g = (kb * DZ_KBLOCK + 64 * j) / P.gs;
-                if (g != gprev) {
-                  s0 = sp[(size_t)g * P.N];
-                  s1 = sp[(size_t)g * P.N + 16];
-                  gprev = g;
-                }
-                A0 *= s0;
-                A1 *= s1;
+                // the lane's operand row is n0 + 16*s + jj; one scale per (row, K-group)
+                const _Float16* sp = P.scales + (size_t)(kd[g] - 1) * P.scales_slot + n0 + jj +
+                                     (size_t)((kb * DZ_KBLOCK + 64 * j) / P.gs) * P.N;
+                A0 *= sp[0];
+                A1 *= sp[16];
               }
-              const int mw = (int)cur.meta[j];
-#pragma unroll
-              for (int tt = 0; tt < TT; ++tt) {
-                if ((dm >> (tt * 16)) & 0xffffull) {
-                  h8_t blo, bhi;
-                  ldsB(tt, j, blo, bhi);
-                  h16_t B = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11,
-                                                    12, 13, 14, 15);
-                  t0[tt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B, t0[tt], mw, 0, 0);
-                  t1[tt] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B, t1[tt], mw, 0, 1);
-                }
-              }
-            }
-#pragma unroll
-            for (int tt = 0; tt < TT; ++tt) {
-              // select, not multiply: columns outside the segment may hold anything
-              accd[0][tt] += in[tt] ? t0[tt] : (f4_t){0.f, 0.f, 0.f, 0.f};
-              accd[1][tt] += in[tt] ? t1[tt] : (f4_t){0.f, 0.f, 0.f, 0.f};
+              const int mw = (int)slot[g].meta[j];
+              t0[g] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B, t0[g], mw, 0, 0);
+              t1[g] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B, t1[g], mw, 0, 1);
             }
           }
+          // keep the steps in program order: hoisting the next steps' operand reads and unpacking
+          // above this point costs more registers than the latency it hides
+          __builtin_amdgcn_sched_barrier(0);
         }
+        // keep only the columns of the delta.  A 0/1 multiplier is enough: a column is computed
+        // from that token's activations alone, so a non-finite value can only come from, and stay
+        // in, the column of the token that supplied it.
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+          const float in = (float)((cols[g] >> jj) & 1u);
+          accd[0][tt] += t0[g] * in;
+          accd[1][tt] += t1[g] * in;
+        }
+      };
+
+      int par = 0;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        unsigned long long m = tile_bits(tt);
+        bool first = true;
+        do {
+          if (par == 0) {
+            consume(tt, ring[0], m, first);
+            load_batch(ring[0]);
+          } else {
+            consume(tt, ring[1], m, first);
+            load_batch(ring[1]);
+          }
+          par ^= 1;
+          first = false;
+        } while (m);
       }
     }
+    if (r == 0) DZ_TS(4);
   }
   DZ_TS(5);
 
@@ -296,6 +314,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   auto part_ptr = [&](int kc2, int item) -> float* {
     return P.partials + (((size_t)kc2 * P.NP + np) * (2 * TT) + item) * 256 + lane;
   };
+
   __syncthreads();  // every wavefront is done with its activations: LDS becomes the buffer
   DZ_TS(6);
   // item = tt*2 + s; red[wave][item][lane]
