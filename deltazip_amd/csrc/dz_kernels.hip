@@ -623,7 +623,7 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
                           size_t workspace_bytes, void* stream) {
   if (!x || !indices || !y) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
-  if (S < 0) return DZ_EINVAL;
+  if (S < 1) return DZ_EINVAL;  // at least one slot: the kernels always address slot 0
   size_t cb, mb, sb;
   int rc = dz_native_sizes(K, N, bits, group_size, &cb, &mb, &sb);
   if (rc) return rc;

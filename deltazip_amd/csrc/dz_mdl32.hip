@@ -3,17 +3,18 @@
 // One workgroup = 4 wavefronts = one n-pair (32 output rows) x a chunk of k-blocks; each
 // wavefront owns whole k-blocks (256 input columns) of that n-pair and is self-sufficient until
 // the final reduction:
-//   * at entry it requests its activations slice (straight into LDS, global_load_lds_dwordx4) and
-//     its 32 x 256 base-weight tile (16 x 128-bit loads per lane), so HBM traffic starts at once;
 //   * the token ids are fetched first; the distinct deltas of the batch are enumerated
 //     with ballots (no sort, no barrier): output columns stay in token order and each delta gets a
 //     per-column mask.  Batches that arrive sorted by id (as the reference's scheduler delivers
 //     them) touch fewer column tiles;
-//   * the packed words of up to 8 deltas (two batches of 4) are then requested together;
-//   * compute runs column tile by column tile: one read of the dense operand (activations, from
-//     the wavefront's own LDS slice) feeds the base product (v_mfma_f32_16x16x32_f16) and the
-//     products of every delta of the current batch (2:4-sparse v_smfmac_f32_16x16x64_f16, unpacked
-//     codes as the sparse operand, stored positions as its index operand);
+//   * then everything else is requested at once, in the order it will be used: activations slice
+//     (straight into LDS), the packed words of up to 8 deltas (two batches of 4), the base tile.
+//     The number of requests is fixed, so the wait in front of each use is exact and the deltas
+//     are multiplied while the base tile is still on its way;
+//   * one read of the dense operand (activations, from the wavefront's own LDS slice) feeds every
+//     delta of the current batch (2:4-sparse v_smfmac_f32_16x16x64_f16, unpacked codes as the
+//     sparse operand, stored positions as its index operand); the base tile follows on
+//     v_mfma_f32_16x16x32_f16;
 //   * partial sums of the 4 wavefronts meet in LDS; when K is split over several workgroups the
 //     per-chunk sums go to a workspace and the last workgroup to arrive adds them in a fixed
 //     order (deterministic) and writes y.
@@ -24,7 +25,7 @@ namespace {
 
 constexpr int WK32 = 4;
 
-template <int BITS, int TT, bool PRE>
+template <int BITS, int TT, bool PRE, bool HAS_BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? 4 : (TT == 2 ? 2 : 3);   // deltas per batch; two batches are in flight
@@ -71,9 +72,9 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   u4_t a[2][4][2];  // base tile: [row fragment][step][half]
 
   // Activations slice of k-block kb -> LDS, rows in token order; rows >= T repeat row T-1 (they
-  // only feed output columns that are never stored).  Then the base tile.  Addresses are a
-  // wavefront-uniform base plus one 32-bit lane offset.
-  auto issue_x_and_base = [&](int kb, int lane_r) {
+  // only feed output columns that are never stored).  Addresses are a wavefront-uniform base plus
+  // one 32-bit lane offset.
+  auto issue_x = [&](int kb, int lane_r) {
     const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
@@ -84,20 +85,20 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
                                        16, 0, 0);
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (P.wb) {
-      const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
-      const unsigned loff = (unsigned)(lane_r & 15) * Kb + (unsigned)(lane_r >> 4) * 16u;
+  };
+  // The 32 x 256 base tile: 16 loads of 16 bytes per lane.
+  auto issue_base = [&](int kb, int lane_r) {
+    const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
+    const unsigned loff = (unsigned)(lane_r & 15) * Kb + (unsigned)(lane_r >> 4) * 16u;
 #pragma unroll
-      for (int s = 0; s < 2; ++s) {
-        const char* ws = wbb + (size_t)(16 * s) * Kb;
+    for (int s = 0; s < 2; ++s) {
+      const char* ws = wbb + (size_t)(16 * s) * Kb;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
-            a[s][j][h] = __builtin_nontemporal_load((const u4_t*)(ws + loff + (128 * j + 64 * h)));
-      }
+        for (int h = 0; h < 2; ++h)
+          a[s][j][h] = __builtin_nontemporal_load((const u4_t*)(ws + loff + (128 * j + 64 * h)));
     }
-    __builtin_amdgcn_sched_barrier(0);
   };
 
   // token ids: lane t keeps the key of token t (0 = base only, id + 1 otherwise, INT_MAX for
@@ -118,87 +119,83 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     int lane_r = lane;
     asm volatile("" : "+v"(lane_r));
 
-    // ---- delta walk.  Visits are (column tile, delta) pairs: tiles in order, inside a tile the
-    // distinct deltas in order of first token.  They are cut into batches of at most G that never
-    // span tiles; every tile gets at least one (possibly empty) batch.  The loader runs two
-    // batches ahead of the consumer; both follow the same rule, with scalar state only.
-    Frag<BITS> ring[2][G];
-    int ld_tt = 0;
-    unsigned long long ld_m = mdelta & 0xffffull;
-    auto tile_bits = [&](int tt) -> unsigned long long { return (mdelta >> (16 * tt)) & 0xffffull; };
-    auto pop = [&](unsigned long long& m, int tt, int& kd, unsigned& cols) {
-      const int l = __builtin_ctzll(m) + 16 * tt;
-      kd = __builtin_amdgcn_readlane(key, l);
-      const unsigned long long dm = (__builtin_amdgcn_ballot_w64(key == kd) >> (16 * tt)) & 0xffffull;
-      m &= ~dm;
-      cols = (unsigned)dm;  // columns of this tile that belong to the delta
-    };
-    auto load_batch = [&](Frag<BITS> (&slot)[G]) {
-      if (ld_tt >= TT) return;
-#pragma unroll
-      for (int g = 0; g < G; ++g)
-        if (ld_m) {
-          int kd;
-          unsigned cols;
-          pop(ld_m, ld_tt, kd, cols);
-          slot[g] = load_frag<BITS>(P, kd - 1, np, kb, lane_r);
-        }
-      if (ld_m == 0) {
-        ++ld_tt;
-        if (ld_tt < TT) ld_m = tile_bits(ld_tt);
-      }
-    };
-
-    // Issue order: packed deltas, activations, base tile.  In round 0 nothing is requested before
-    // the ids are in: a request queued behind this kernel's own flood of weight loads would take
-    // far longer than the ids do on an idle memory system, and the packed deltas depend on them.
     if (r == 0) {
+      // nothing is requested before the ids are in (see above)
       if (lane < P.T) {
         key = (id < 0 || id >= P.S) ? 0 : (int)id + 1;
         if ((id < -1 || id >= P.S) && blockIdx.x == 0 && wave == 0) atomicOr(P.status, 1u);
       }
       // tokens that carry a delta; lanes >= T never match
       mdelta = __builtin_amdgcn_ballot_w64(key != 0 && key != 0x7fffffff);
-      ld_m = mdelta & 0xffffull;
       DZ_TS(1);
     }
-    if (active) {
-      load_batch(ring[0]);
-      load_batch(ring[1]);
-    }
+    if (!active) continue;
+
+    // ---- delta walk (scalar state only).  The distinct deltas of the batch are visited in order
+    // of their first token, G at a time; `pop` takes the next one and returns the output columns
+    // (tokens) that belong to it.  The loader runs two batches ahead of the consumer.
+    Frag<BITS> ring[2][G];
+    unsigned long long ld_m = mdelta, use_m = mdelta;
+    auto pop = [&](unsigned long long& m, int& kd, unsigned long long& cols) {
+      const int l = __builtin_ctzll(m);
+      kd = __builtin_amdgcn_readlane(key, l);
+      cols = __builtin_amdgcn_ballot_w64(key == kd);
+      m &= ~cols;
+    };
+    // Always G requests, so that the number of loads in flight is known at compile time and the
+    // waits in front of each use can be exact: a slot without a delta re-reads 16 bytes.
+    auto load_batch = [&](Frag<BITS> (&slot)[G]) {
+#pragma unroll
+      for (int g = 0; g < G; ++g) {
+        int kd = 1;
+        unsigned long long cols;
+        const bool real = ld_m != 0;
+        if (real) pop(ld_m, kd, cols);
+        slot[g] = load_frag<BITS>(P, kd - 1, np, kb, real ? lane_r : 0);
+      }
+    };
+
+    // ---- issue order: activations (L2 -> LDS), packed deltas of two batches, base tile
+    issue_x(kb, lane_r);
+    load_batch(ring[0]);
+    load_batch(ring[1]);
     __builtin_amdgcn_sched_barrier(0);
-    if (active) issue_x_and_base(kb, lane_r);
+    if (HAS_BASE) issue_base(kb, lane_r);
     __builtin_amdgcn_sched_barrier(0);
     if (r == 0) DZ_TS(2);
-    // Loads return in order and the base tile (16 loads) was requested last: once at most 16 loads
-    // are outstanding, the packed deltas and this wavefront's LDS slice are complete.  (The
-    // compiler does not order LDS reads after LDS-direct loads by itself.)
-    if (P.wb) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // Loads return in order and the activations were requested first: once only the loads issued
+    // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
+    // not order LDS reads after LDS-direct loads by itself.)
+    {
+      constexpr int later = 2 * G * (BITS == 2 ? 2 : 3) + (HAS_BASE ? 16 : 0);
+      // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
+      __builtin_amdgcn_s_waitcnt((later & 15) | (7 << 4) | (15 << 8) | ((later >> 4) << 14));
+      asm volatile("" ::: "memory");
+    }
     __builtin_amdgcn_sched_barrier(0);
     if (r == 0) DZ_TS(3);
 
-    if (active) {
-      auto ldsB = [&](int tt, int j, h8_t& lo, h8_t& hi) {
-        const char* p = (const char*)xw + (j >> 1) * 256;
-        lo = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 0]);
-        hi = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 1]);
-      };
-      // one batch of one column tile: every operand read feeds the base product (first batch of
-      // the tile only) and all deltas of the batch
-      auto consume = [&](int tt, Frag<BITS> (&slot)[G], unsigned long long& m, bool with_base) {
-        int kd[G];
-        unsigned cols[G];
-        int nb = 0;
+    auto ldsB = [&](int tt, int j, h8_t& lo, h8_t& hi) {
+      const char* p = (const char*)xw + (j >> 1) * 256;
+      lo = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 0]);
+      hi = *(const h8_t*)(p + boff[tt][(j & 1) * 2 + 1]);
+    };
+    // one batch: for every column tile that holds tokens of these deltas, one pass over the four
+    // steps in which each operand read feeds all deltas of the batch
+    auto consume = [&](Frag<BITS> (&slot)[G]) {
+      int kd[G];
+      unsigned long long cols[G];
+      unsigned long long any = 0;
 #pragma unroll
-        for (int g = 0; g < G; ++g) {
-          kd[g] = 0;
-          cols[g] = 0;
-          if (m) {
-            pop(m, tt, kd[g], cols[g]);
-            nb = g + 1;
-          }
-        }
+      for (int g = 0; g < G; ++g) {
+        kd[g] = 1;
+        cols[g] = 0;
+        if (use_m) pop(use_m, kd[g], cols[g]);
+        any |= cols[g];
+      }
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        if (((any >> (16 * tt)) & 0xffffull) == 0) continue;
         f4_t t0[G], t1[G];
 #pragma unroll
         for (int g = 0; g < G; ++g) {
@@ -209,21 +206,11 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
         for (int j = 0; j < 4; ++j) {
           h8_t blo, bhi;
           ldsB(tt, j, blo, bhi);
-          if (with_base && P.wb) {
-#pragma unroll
-            for (int s = 0; s < 2; ++s) {
-              H8U a0, a1;
-              a0.v = a[s][j][0];
-              a1.v = a[s][j][1];
-              accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0.h, blo, accb[s][tt], 0, 0, 0);
-              accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1.h, bhi, accb[s][tt], 0, 0, 0);
-            }
-          }
           const h16_t B = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12,
                                                   13, 14, 15);
 #pragma unroll
           for (int g = 0; g < G; ++g) {
-            if (g < nb) {
+            if ((cols[g] >> (16 * tt)) & 0xffffull) {
               h8_t A0, A1;
               if (BITS == 2) {
                 unpack2(slot[g].code[0][j], MAGIC, A0, A1);
@@ -247,35 +234,53 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
           // above this point costs more registers than the latency it hides
           __builtin_amdgcn_sched_barrier(0);
         }
-        // keep only the columns of the delta.  A 0/1 multiplier is enough: a column is computed
+        // keep only the columns of each delta.  A 0/1 multiplier is enough: a column is computed
         // from that token's activations alone, so a non-finite value can only come from, and stay
         // in, the column of the token that supplied it.
 #pragma unroll
         for (int g = 0; g < G; ++g) {
-          const float in = (float)((cols[g] >> jj) & 1u);
+          const float in = (float)((unsigned)(cols[g] >> (16 * tt + jj)) & 1u);
           accd[0][tt] += t0[g] * in;
           accd[1][tt] += t1[g] * in;
         }
-      };
+      }
+    };
 
-      int par = 0;
+    // first two batches in straight-line code; their data arrives before the base tile does
+    consume(ring[0]);
+    if (ld_m) load_batch(ring[0]);
+    consume(ring[1]);
+    if (ld_m) load_batch(ring[1]);
+    // ---- base: dense matrix-core product over all token tiles
+    if (HAS_BASE) {
 #pragma unroll
-      for (int tt = 0; tt < TT; ++tt) {
-        unsigned long long m = tile_bits(tt);
-        bool first = true;
-        do {
-          if (par == 0) {
-            consume(tt, ring[0], m, first);
-            load_batch(ring[0]);
-          } else {
-            consume(tt, ring[1], m, first);
-            load_batch(ring[1]);
+      for (int tt = 0; tt < TT; ++tt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          h8_t blo, bhi;
+          ldsB(tt, j, blo, bhi);
+#pragma unroll
+          for (int s = 0; s < 2; ++s) {
+            H8U a0, a1;
+            a0.v = a[s][j][0];
+            a1.v = a[s][j][1];
+            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0.h, blo, accb[s][tt], 0, 0, 0);
+            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1.h, bhi, accb[s][tt], 0, 0, 0);
           }
-          par ^= 1;
-          first = false;
-        } while (m);
+        }
+    }
+    // more than 2*G deltas: keep going, two batches per turn
+    while (use_m) {
+      consume(ring[0]);
+      if (ld_m) load_batch(ring[0]);
+      if (use_m) {
+        consume(ring[1]);
+        if (ld_m) load_batch(ring[1]);
       }
     }
+    // Every load of this round has been consumed by now; saying so keeps the waits of the next
+    // round exact (the compiler would otherwise assume refill loads may still be pending).
+    __builtin_amdgcn_s_waitcnt(0 | (7 << 4) | (15 << 8));
     if (r == 0) DZ_TS(4);
   }
   DZ_TS(5);
@@ -388,24 +393,21 @@ int launch32(MdlParams P, bool pre, hipStream_t st, int ksplit_override) {
   P.nsplit = (P.NKB + P.cb - 1) / P.cb;
   const int grid = (P.NP + 7) / 8 * 8 * P.nsplit;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
-  static bool attr_done[2] = {false, false};
-  if (pre) {
-    auto kern = dz_mdl32_kernel<BITS, TT, true>;
-    if (!attr_done[1]) {
+  static bool attr_done[4] = {false, false, false, false};
+  const bool has_base = P.wb != nullptr;
+  auto go = [&](auto kern, int slot) -> int {
+    if (!attr_done[slot]) {
       if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
         return DZ_ELAUNCH;
-      attr_done[1] = true;
+      attr_done[slot] = true;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, P);
-  } else {
-    auto kern = dz_mdl32_kernel<BITS, TT, false>;
-    if (!attr_done[0]) {
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return DZ_ELAUNCH;
-      attr_done[0] = true;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, P);
-  }
+    return DZ_OK;
+  };
+  int rc;
+  if (pre) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, true, true>, 0) : go(dz_mdl32_kernel<BITS, TT, true, false>, 1);
+  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, false, true>, 2) : go(dz_mdl32_kernel<BITS, TT, false, false>, 3);
+  if (rc) return rc;
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
