@@ -33,6 +33,12 @@ SHAPES = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096)
 T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1
 
 
+# HBM bytes per launch (average over the 7 launches of a step) of the default workload, from
+# rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what the same counter
+# reads for the --calib-copy-mib copy kernel; the figures are in profiles/*__hbm_traffic.txt.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 123460880
+
+
 def algorithmic_bytes(K, N, T, bits, d_present, G=1):
     """Bytes one layer call has to move: base fp16 once; per distinct delta present its codes
     (kept half, `bits` each), a 2-bit position per kept value and the fp16 scales; activations in,
@@ -118,6 +124,9 @@ def main():
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ksplit", type=int, default=0)
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="before the timed region, run a plain elementwise copy kernel over this many MiB "
+                         "(reads and writes that much): the yardstick for scaling FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -171,6 +180,14 @@ def main():
             if rc:
                 raise RuntimeError(f"dz_multi_delta_linear failed: {lib.dz_strerror(rc).decode()}")
 
+    if args.calib_copy_mib > 0:
+        src = torch.ones(args.calib_copy_mib << 19, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)         # one elementwise kernel: reads src once, writes dst once
+        torch.cuda.synchronize()
+        del src, dst
+
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
@@ -184,6 +201,7 @@ def main():
     wall = time.perf_counter() - t0
     gpu_s = e0.elapsed_time(e1) * 1e-3
 
+    default_workload = not args.unsorted and args.ksplit == 0
     launches = args.steps * len(SHAPES)
     step_bytes = sum(algorithmic_bytes(K, N, T, BITS, d_present) for _, K, N in SHAPES)
     avg_launch_s = gpu_s / launches              # includes the gaps between consecutive launches
@@ -221,7 +239,8 @@ def main():
         "us_per_layer_call": round(avg_launch_s * 1e6, 2),
         "per_shape": per_call_us,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
                      "kernel": "dz_mdl32_kernel<2,2,false>",
                      "algorithmic_bytes_per_launch": step_bytes // len(SHAPES),
                      "avg_launch_us": round(avg_launch_s * 1e6, 2)},
