@@ -46,21 +46,6 @@ def algorithmic_bytes(K, N, T, bits, d_present, G=1):
     return 2 * K * N + d_present * (K * N * bits // 16 + K * N // 8 + 2 * G * N) + 2 * T * K + 2 * T * N + 8 * T
 
 
-def random_native_stack(K, N, bits, gs, nd, dev, gen):
-    """Random deltas directly in the native layout (valid 2:4 positions), on the GPU."""
-    from deltazip_amd import ops
-    qs, ms, ss = ops.stacked_shapes(K, N, bits, gs)
-    q = torch.randint(-2 ** 31, 2 ** 31 - 1, (nd,) + qs, dtype=torch.int32, device=dev, generator=gen)
-    pairs = torch.tensor([0b0100, 0b1000, 0b1100, 0b1001, 0b1101, 0b1110], dtype=torch.int64, device=dev)
-    nwords = nd * ms[0] * ms[1] // 2
-    w = torch.zeros(nwords, dtype=torch.int64, device=dev)
-    for f in range(8):
-        w |= pairs[torch.randint(0, 6, (nwords,), device=dev, generator=gen)] << (4 * f)
-    m = torch.where(w >= 2 ** 31, w - 2 ** 32, w).to(torch.int32).view(torch.int16).view((nd,) + ms)
-    s = (torch.rand((nd,) + ss, device=dev, generator=gen) * 1e-3 + 2e-4).half()
-    return q, m, s
-
-
 def parity_check(dev):
     """Small same-run parity gate against the CPU oracle: dequant bit-exact, output rel err."""
     from oracle import dz_oracle as o
@@ -135,6 +120,7 @@ def main():
         print("bench.py needs a GPU (there is no CPU fallback for the measured path)", file=sys.stderr)
         sys.exit(2)
     from deltazip_amd import _lib, ops
+    from deltazip_amd.synthetic import random_native_stack
     lib = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
