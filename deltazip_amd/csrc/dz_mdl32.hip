@@ -169,7 +169,9 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     {
       constexpr int later = 2 * G * (BITS == 2 ? 2 : 3) + (HAS_BASE ? 16 : 0);
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
-      __builtin_amdgcn_s_waitcnt((later & 15) | (7 << 4) | (15 << 8) | ((later >> 4) << 14));
+      // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
+      // believes one outstanding, turns every later vmcnt wait into vmcnt(0)
+      __builtin_amdgcn_s_waitcnt((later & 15) | (7 << 4) | (0 << 8) | ((later >> 4) << 14));
       asm volatile("" ::: "memory");
     }
     __builtin_amdgcn_sched_barrier(0);
