@@ -30,7 +30,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 SHAPES = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096), ("o_proj", 4096, 4096),
           ("gate_proj", 4096, 11008), ("up_proj", 4096, 11008), ("down_proj", 11008, 4096)]   # (name, K, N)
-T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1
+T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1    # the default workload (configuration 2)
 
 
 # HBM bytes per launch (average over the 7 launches of a step) of the default workload, from
@@ -100,12 +100,49 @@ def cpu_baseline():
             "seconds_per_step": total, "seconds_per_shape": per_shape, "os_cpu_count": os.cpu_count()}
 
 
+SHAPES_13B = [("q_proj", 5120, 5120), ("k_proj", 5120, 5120), ("v_proj", 5120, 5120), ("o_proj", 5120, 5120),
+              ("gate_proj", 5120, 13824), ("up_proj", 5120, 13824), ("down_proj", 13824, 5120)]
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+# BASELINE.json's configurations.  The default (and the one the metric is quoted on) is 2; the
+# others are parity-test cases that can also be timed here with --config.
+CONFIGS = {
+    1: dict(name="4096->4096, 1 token, one 4-bit delta (per-channel scales)", shapes=[("linear", 4096, 4096)],
+            T=1, S=1, bits=4, gs=-1, ids="zeros", bound="hbm"),
+    2: dict(name="Llama-2-7B decode projections (q,k,v,o 4096->4096; gate,up 4096->11008; down 11008->4096), "
+                 "one step = these 7 multi-delta linear calls; 32 tokens, 8 deltas (2-bit, 2:4 sparse, "
+                 "per-channel fp16 scales), ids uniform over the deltas",
+            shapes=SHAPES, T=32, S=8, bits=2, gs=-1, ids="uniform", bound="hbm"),
+    3: dict(name="Llama-2-7B projections, 64 tokens, 32 deltas (4-bit, 2:4, group size 128), Zipf(1.5) ids",
+            shapes=SHAPES, T=64, S=32, bits=4, gs=128, ids="zipf", bound="hbm"),
+    4: dict(name="Llama-2-13B prefill projections, 16 requests x 512 tokens, each bound to its own delta "
+                 "(2-bit, 2:4, per-channel)", shapes=SHAPES_13B, T=8192, S=16, bits=2, gs=-1, ids="blocks",
+            bound="mfma"),
+    5: dict(name="Llama-2-7B decode projections, 128 tokens, 64 resident deltas (2-bit, 2:4, per-channel), "
+                 "ids uniform", shapes=SHAPES, T=128, S=64, bits=2, gs=-1, ids="uniform", bound="hbm"),
+}
+
+
+def make_ids(kind, t, s, dev, gen, sort):
+    if kind == "zeros":
+        return torch.zeros(t, dtype=torch.int64, device=dev)
+    if kind == "blocks":
+        return torch.repeat_interleave(torch.arange(s, device=dev), t // s)
+    if kind == "zipf":
+        p = torch.arange(1, s + 1, device=dev, dtype=torch.float32) ** -1.5
+        ids = torch.multinomial(p / p.sum(), t, replacement=True, generator=gen)
+    else:
+        ids = torch.randint(0, s, (t,), device=dev, generator=gen)
+    return torch.sort(ids).values if sort else ids   # the serving scheduler delivers batches sorted by delta id
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--layers", type=int, default=4, help="distinct decoder layers kept in HBM and visited in turn")
+    ap.add_argument("--steps", type=int, default=0, help="timed steps (default 200; 10 for --config 4)")
+    ap.add_argument("--warmup", type=int, default=0, help="untimed steps (default 20; 2 for --config 4)")
+    ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS), help="BASELINE.json configuration")
+    ap.add_argument("--layers", type=int, default=0, help="distinct decoder layers kept in HBM and visited in turn")
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ksplit", type=int, default=0)
@@ -121,6 +158,11 @@ def main():
         sys.exit(2)
     from deltazip_amd import _lib, ops
     from deltazip_amd.synthetic import random_native_stack
+    cfg = CONFIGS[args.config]
+    shapes, T, S, bits, gs = cfg["shapes"], cfg["T"], cfg["S"], cfg["bits"], cfg["gs"]
+    steps = args.steps or (10 if args.config == 4 else 200)
+    warmup = args.warmup or (2 if args.config == 4 else 20)
+    nlayers = args.layers or {1: 16, 2: 4, 3: 2, 4: 1, 5: 2}[args.config]
     lib = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -129,42 +171,50 @@ def main():
     parity = parity_check(dev)
 
     # ---- resident inputs
-    ids = torch.randint(0, NUM_DELTAS, (T,), device=dev, generator=gen)
-    if not args.unsorted:
-        ids = torch.sort(ids).values            # the serving scheduler delivers batches sorted by delta id
+    ids = make_ids(cfg["ids"], T, S, dev, gen, not args.unsorted)
     d_present = int(torch.unique(ids).numel())
     layers = []
-    for _ in range(args.layers):
+    for _ in range(nlayers):
         calls = []
-        for name, K, N in SHAPES:
-            q, m, s = random_native_stack(K, N, BITS, GROUP, NUM_DELTAS, dev, gen)
+        for name, K, N in shapes:
+            q, m, s = random_native_stack(K, N, bits, gs, S, dev, gen)
             wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
             x = torch.randn((T, K), device=dev, generator=gen).half()
             y = torch.empty((T, N), dtype=torch.float16, device=dev)
             calls.append((name, K, N, x, wb, q, m, s, y))
         layers.append(calls)
-    ws_bytes = max(lib.dz_workspace_bytes(T, K, N) for _, K, N in SHAPES)
-    ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
     stream = torch.cuda.current_stream().cuda_stream
     ops.set_ksplit(args.ksplit)
+    fused = T <= 128
 
-    # pre-marshalled C-ABI calls (device pointers and sizes only)
-    f = lib.dz_multi_delta_linear
-    vp = C.c_void_p
-    prepared = []
-    for calls in layers:
-        pc = []
-        for name, K, N, x, wb, q, m, s, y in calls:
-            pc.append((vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
-                       vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, NUM_DELTAS, BITS, GROUP, 0, N,
-                       vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream)))
-        prepared.append(pc)
+    if fused:
+        # pre-marshalled C-ABI calls (device pointers and sizes only)
+        ws_bytes = max(lib.dz_workspace_bytes(T, K, N) for _, K, N in shapes)
+        ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
+        f = lib.dz_multi_delta_linear
+        vp = C.c_void_p
+        prepared = []
+        for calls in layers:
+            pc = []
+            for name, K, N, x, wb, q, m, s, y in calls:
+                pc.append((vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
+                           vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
+                           vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream)))
+            prepared.append(pc)
 
-    def step(i):
-        for a in prepared[i % len(prepared)]:
-            rc = f(*a)
+        def call(i, idx):
+            rc = f(*prepared[i % len(prepared)][idx])
             if rc:
                 raise RuntimeError(f"dz_multi_delta_linear failed: {lib.dz_strerror(rc).decode()}")
+    else:
+        # prefill-sized: the host wrapper segments the batch and runs dequant + pair-GEMM per delta
+        def call(i, idx):
+            name, K, N, x, wb, q, m, s, y = layers[i % len(layers)][idx]
+            ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y)
+
+    def step(i):
+        for idx in range(len(shapes)):
+            call(i, idx)
 
     if args.calib_copy_mib > 0:
         src = torch.ones(args.calib_copy_mib << 19, dtype=torch.float16, device=dev)
@@ -174,65 +224,80 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         step(i)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()                                  # on the stream the kernels are launched on
-    for i in range(args.steps):
+    for i in range(steps):
         step(i)
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     gpu_s = e0.elapsed_time(e1) * 1e-3
 
-    default_workload = not args.unsorted and args.ksplit == 0
-    launches = args.steps * len(SHAPES)
-    step_bytes = sum(algorithmic_bytes(K, N, T, BITS, d_present) for _, K, N in SHAPES)
+    def abytes(K, N):
+        return algorithmic_bytes(K, N, T, bits, d_present, 1 if gs == -1 else K // gs)
+    default_workload = args.config == 2 and not args.unsorted and args.ksplit == 0
+    launches = steps * len(shapes)
+    step_bytes = sum(abytes(K, N) for _, K, N in shapes)
+    step_flops = sum(2.0 * T * K * N for _, K, N in shapes)
     avg_launch_s = gpu_s / launches              # includes the gaps between consecutive launches
-    achieved = (step_bytes / len(SHAPES)) / avg_launch_s / 1e9
-    ms_per_step = wall / args.steps * 1e3
+    ms_per_step = wall / steps * 1e3
 
-    # per-shape kernel time (event pairs around single launches, outside the timed region)
+    # per-shape time (event pairs around single calls, outside the timed region)
     per_call_us = {}
-    for name, K, N in (("4096x4096", 4096, 4096), ("4096x11008", 4096, 11008), ("11008x4096", 11008, 4096)):
-        idx = [j for j, sh in enumerate(SHAPES) if (sh[1], sh[2]) == (K, N)][0]
+    for (K, N) in dict.fromkeys((K, N) for _, K, N in shapes):
+        idx = [j for j, sh in enumerate(shapes) if (sh[1], sh[2]) == (K, N)][0]
         ts = []
-        for i in range(12):
-            a = prepared[i % len(prepared)][idx]
+        for i in range(12 if fused else 4):
             s0, s1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            s0.record(); f(*a); s1.record(); torch.cuda.synchronize()
+            s0.record(); call(i, idx); s1.record(); torch.cuda.synchronize()
             ts.append(s0.elapsed_time(s1) * 1e3)
         us = float(np.median(ts[2:]))
-        b = algorithmic_bytes(K, N, T, BITS, d_present)
-        per_call_us[name] = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 3)}
+        b = abytes(K, N)
+        ent = {"us": round(us, 2), "GBps": round(b / us / 1e3, 1), "frac": round(b / us / 1e3 / HBM_PEAK_GBPS, 3)}
+        if cfg["bound"] == "mfma":
+            ent = {"us": round(us, 2), "TFLOPs": round(2.0 * T * K * N / us / 1e6, 1),
+                   "frac": round(2.0 * T * K * N / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3)}
+        per_call_us[f"{K}x{N}"] = ent
+
+    if cfg["bound"] == "hbm":
+        achieved = (step_bytes / len(shapes)) / avg_launch_s / 1e9
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
+                    "kernel": "dz_mdl32_kernel" if T <= 32 else "dz_mdl_kernel",
+                    "algorithmic_bytes_per_launch": step_bytes // len(shapes),
+                    "avg_launch_us": round(avg_launch_s * 1e6, 2)}
+    else:
+        # base contraction only (2*T*K*N per call); the per-delta dequantisation and the delta half of
+        # the pair-GEMM are extra work inside the same time
+        achieved = (step_flops / len(shapes)) / avg_launch_s / 1e12
+        roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                    "kernel": "dz_gemm_kernel (pair)", "algorithmic_flops_per_call": step_flops / len(shapes),
+                    "avg_call_us": round(avg_launch_s * 1e6, 2)}
 
     out = {
         "metric": "multi-delta linear tokens/s + achieved HBM TB/s (% peak), Llama-7B shapes",
         "value": T / (ms_per_step * 1e-3),
         "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "Llama-2-7B decode projections (q,k,v,o 4096->4096; gate,up 4096->11008; "
-                               "down 11008->4096), one step = these 7 multi-delta linear calls; 32 tokens, "
-                               "8 deltas (2-bit, 2:4 sparse, per-channel fp16 scales), ids uniform over the deltas"
-                               + ("" if args.unsorted else ", batch sorted by delta id"),
-                   "tokens": T, "deltas": NUM_DELTAS, "deltas_present": d_present, "bits": BITS,
-                   "layers_resident": args.layers, "launches_per_step": len(SHAPES)},
+        "config": {"workload": cfg["name"] + ("" if args.unsorted or cfg["ids"] in ("zeros", "blocks")
+                                              else ", batch sorted by delta id"),
+                   "baseline_config": args.config, "tokens": T, "deltas": S, "deltas_present": d_present,
+                   "bits": bits, "group_size": gs, "layers_resident": nlayers, "launches_per_step": len(shapes)},
         "us_per_layer_call": round(avg_launch_s * 1e6, 2),
         "per_shape": per_call_us,
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
-                     "kernel": "dz_mdl32_kernel<2,2,false>",
-                     "algorithmic_bytes_per_launch": step_bytes // len(SHAPES),
-                     "avg_launch_us": round(avg_launch_s * 1e6, 2)},
+        "roofline": roofline,
         "parity": parity,
     }
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and args.config == 2:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
 

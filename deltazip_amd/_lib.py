@@ -27,6 +27,7 @@ SIGNATURES = {
                                    _vp, _sz, _vp]),
     "dz_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16_pair": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "dz_gemm_f16_grouped": (_i, [_vp, _vp, _vp, C.c_longlong, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_set_ksplit": (None, [_i]),
 }
 

@@ -1,5 +1,17 @@
-// Dense fp16 GEMM on the gfx950 matrix cores: y[T, N] (+)= x[T, K] @ w[N, K]^T, fp32 accumulate.
-// Used for the base product at prefill-sized token counts.
+// Dense fp16 GEMM on the gfx950 matrix cores for prefill-sized token counts:
+//   y[t, :] (+)= x[t, :] @ w^T  (+ x[t, :] @ w2[g(t)]^T),   fp32 accumulation, fp16 in and out.
+// The optional second weight differs per block of rows ("grouped"): the rows are tokens sorted by
+// delta id, w is the base weight and w2[g] the dequantised delta of group g, and both products
+// share the fp32 accumulators, so base and delta are never added in fp16.
+//
+// One workgroup (4 wavefronts, 2 x 2) computes a 256 (tokens) x 256 (output features) tile; each
+// wavefront owns 128 x 128 of it as 4 x 4 v_mfma_f32_32x32x16_f16 tiles (256 accumulator
+// registers).  K is walked in slabs of 64: both operand slabs (2 x 32 KiB) go from global memory
+// straight into LDS (LDS-direct loads, 16 bytes per lane) into one of two buffers, so the next
+// slab is on its way while the matrix cores work on the current one; one barrier per slab.
+// Operand rows in LDS are 128 bytes; the 16-byte chunk index is XOR-ed with half the row number,
+// which keeps the 32-row fragment reads off shared banks.  Workgroups are numbered so that the 32 that run
+// together on one XCD form a 4 x 8 block of tiles and share operand slabs in that XCD's L2.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -11,124 +23,197 @@ typedef float f16_t __attribute__((ext_vector_type(16)));
 
 namespace {
 
-// Workgroup tile 128 (tokens) x 128 (outputs), 4 wavefronts in 2 x 2, each 64 x 64 as 2 x 2
-// v_mfma_f32_32x32x16_f16 tiles.  Both operands are K-contiguous, so every lane's 8 halves of an
-// operand are one 16-byte load.  Tiles are staged through LDS in 64-column slabs.
-constexpr int TM = 128, TN = 128, TK = 64;
-constexpr int LDS_STRIDE = TK + 8;  // halves; the pad keeps 16-byte row reads off shared banks
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int SLAB = 256 * BK * 2;        // bytes of one operand slab in LDS
+constexpr int GM = 4, GN = 8;             // tiles per XCD block
 
-// With w2 != nullptr the contraction runs over both weights, y = x @ w^T + x @ w2^T, in the same
-// fp32 accumulators (base weight and a dequantised delta, never summed in fp16).
-__global__ __launch_bounds__(256) void dz_gemm_kernel(const _Float16* __restrict__ x,
-                                                      const _Float16* __restrict__ w,
-                                                      const _Float16* __restrict__ w2,
-                                                      _Float16* __restrict__ y, int T, int K, int N,
-                                                      int accumulate, int ldy) {
-  __shared__ __attribute__((aligned(16))) _Float16 sa[TM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) _Float16 sb[TN * LDS_STRIDE];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+struct GemmParams {
+  const _Float16* x;
+  const _Float16* w;             // first weight [N, K], or nullptr (second product only)
+  const _Float16* w2;            // stack of second weights or nullptr
+  long long w2_stride;           // elements between consecutive second weights
+  const dz_gemm_tile* tiles;     // row blocks, or nullptr: blocks of 256 rows, second weight 0
+  _Float16* y;
+  int T, K, N, accumulate, ldy, tiles_m, tiles_n;
+};
+
+__global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2 buffers][w slab | x slab]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  // XCD-aware tile order: consecutive workgroups land on different XCDs, so give each XCD a
-  // contiguous band of token tiles to keep its share of x and w hot in its own L2
-  const int tiles_n = N / TN;
-  const int tiles_m = (T + TM - 1) / TM;
-  const int total = tiles_m * tiles_n;
-  const int per_xcd = (total + 7) / 8;
-  const int lin = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (lin >= total) return;
-  const int tm = lin / tiles_n, tn = lin % tiles_n;
-  const int m0 = tm * TM, n0 = tn * TN;
 
-  f16_t acc[2][2];
-#pragma unroll
-  for (int a = 0; a < 2; ++a)
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[a][b][r] = 0.f;
+  // workgroup -> tile: XCD-local blocks of GM x GN tiles
+  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+  const int sbn = (P.tiles_n + GN - 1) / GN;
+  const int sb = (q / (GM * GN)) * 8 + xcd, r = q % (GM * GN);
+  const int tm = (sb / sbn) * GM + r / GN, tn = (sb % sbn) * GN + r % GN;
+  if (tm >= P.tiles_m || tn >= P.tiles_n) return;
+  int row_lo = tm * BM, row_hi = min(P.T, row_lo + BM), widx = 0;   // no table: one group, second weight 0
+  if (P.tiles) {
+    row_lo = P.tiles[tm].row_lo;
+    row_hi = P.tiles[tm].row_hi;
+    widx = P.tiles[tm].group;
+  }
+  const int n0 = tn * BN;
+  const _Float16* w2 = (P.w2 && widx >= 0) ? P.w2 + (size_t)widx * P.w2_stride : nullptr;
+  const int nslab1 = P.K / BK, nslab = w2 ? 2 * nslab1 : nslab1;
+  const int s_begin = P.w ? 0 : nslab1;   // no first weight: second product only
+  if (s_begin >= nslab) return;           // neither: the tile is left as it is
+  const unsigned Kb = (unsigned)P.K * 2u;
 
-  const int li = lane & 31, lh = lane >> 5;
-  const int npass = w2 ? 2 : 1;
-  for (int pass = 0; pass < npass; ++pass) {
-  const _Float16* wp = pass ? w2 : w;
-  for (int k0 = 0; k0 < K; k0 += TK) {
-    // stage: 128 rows x 64 halves per operand = 1024 chunks of 16 bytes, 4 per thread
+  f16_t acc[4][4];
 #pragma unroll
-    for (int it = 0; it < 4; ++it) {
-      const int c = it * 256 + tid, row = c >> 3, ch = c & 7;
-      h8_t va = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (m0 + row < T) va = *(const h8_t*)(x + (size_t)(m0 + row) * K + k0 + ch * 8);
-      *(h8_t*)(sa + row * LDS_STRIDE + ch * 8) = va;
-      const h8_t vb = *(const h8_t*)(wp + (size_t)(n0 + row) * K + k0 + ch * 8);
-      *(h8_t*)(sb + row * LDS_STRIDE + ch * 8) = vb;
-    }
-    __syncthreads();
+  for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int kk = 0; kk < TK; kk += 16) {
-      h8_t fa[2], fb[2];
+    for (int b = 0; b < 4; ++b)
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
-        fa[a] = *(const h8_t*)(sa + (wm * 64 + a * 32 + li) * LDS_STRIDE + kk + 8 * lh);
+      for (int e = 0; e < 16; ++e) acc[a][b][e] = 0.f;
+
+  // ---- slab loader: 64 requests of 1 KiB (8 rows x 128 bytes) per slab pair, 16 per wavefront.
+  // Lane l fills LDS row l/8, physical chunk l%8 with global chunk (l%8) ^ ((row >> 1) & 7): a
+  // 16-byte read is served 16 lanes (256 bytes, two rows' worth of banks) per cycle, and 16
+  // consecutive rows then fall on 16 different bank groups.
+  const int lr = lane >> 3;
+  unsigned goff[16];   // global byte offset of this lane's row start + chunk, per request
 #pragma unroll
-      for (int b = 0; b < 2; ++b)
-        fb[b] = *(const h8_t*)(sb + (wn * 64 + b * 32 + li) * LDS_STRIDE + kk + 8 * lh);
-      // operand order (w, x): result rows = output features, columns = tokens, so each lane
-      // ends up with 4 consecutive output features of one token = one 8-byte store
-#pragma unroll
-      for (int a = 0; a < 2; ++a)
-#pragma unroll
-        for (int b = 0; b < 2; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[b], fa[a], acc[a][b], 0, 0, 0);
-    }
-    __syncthreads();
+  for (int i = 0; i < 16; ++i) {
+    const int rq = wave * 16 + i, sub = rq & 31, R = sub * 8 + lr;
+    unsigned rowoff;
+    if (rq < 32) rowoff = (unsigned)min(n0 + R, P.N - 1);           // weight rows (clamped: never stored)
+    else rowoff = (unsigned)min(row_lo + R, row_hi - 1);            // token rows
+    const int lc = (lane & 7) ^ ((R >> 1) & 7);
+    goff[i] = rowoff * Kb + (unsigned)lc * 16u;
   }
+  auto issue = [&](int s, int buf) {
+    const bool second = s >= nslab1;
+    const char* wsrc = (const char*)(second ? w2 : P.w) + (size_t)(second ? s - nslab1 : s) * (BK * 2);
+    const char* xsrc = (const char*)P.x + (size_t)(second ? s - nslab1 : s) * (BK * 2);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int rq = wave * 16 + i, sub = rq & 31;
+      const char* src = (rq < 32 ? wsrc : xsrc) + goff[i];
+      unsigned char* dst = smem + buf * (2 * SLAB) + (rq < 32 ? 0 : SLAB) + sub * 1024;
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    }
+  };
+
+  // ---- fragment addresses: lane (i = lane % 32, g = lane / 32) reads row i of a 32-row tile,
+  // chunk 2*kk + g of the slab row
+  const int li = lane & 31, lg = lane >> 5;
+  int foff[4];   // byte offset inside a slab row for the four k-steps, before adding the row
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) foff[kk] = (((2 * kk + lg) ^ ((li >> 1) & 7)) << 4);
+  const int wrow = (wn * 128 + li) * 128, xrow = (wm * 128 + li) * 128;
+
+  issue(s_begin, s_begin & 1);
+  for (int s = s_begin; s < nslab; ++s) {
+    const int buf = s & 1;
+    // the slab of this turn has been requested one turn ago: wait for this wavefront's share,
+    // then meet the others (their shares are in, and nobody still reads the buffer filled next)
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+    __syncthreads();
+    if (s + 1 < nslab) issue(s + 1, buf ^ 1);
+    const unsigned char* wb = smem + buf * (2 * SLAB);
+    const unsigned char* xb = wb + SLAB;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      h8_t fw[4], fx[4];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 32 * 128 + foff[kk]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 32 * 128 + foff[kk]);
+      // operand order (w, x): result rows = output features, columns = tokens, so each lane ends
+      // up with 4 consecutive output features of one token = one 8-byte store
+#pragma unroll
+      for (int a = 0; a < 4; ++a)
+#pragma unroll
+        for (int b = 0; b < 4; ++b)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[a], fx[b], acc[a][b], 0, 0, 0);
+    }
   }
+
 #pragma unroll
-  for (int a = 0; a < 2; ++a) {
-    const int tok = m0 + wm * 64 + a * 32 + li;
-    if (tok >= T) continue;
+  for (int b = 0; b < 4; ++b) {
+    const int tok = row_lo + wm * 128 + b * 32 + li;
+    if (tok >= row_hi) continue;
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int a = 0; a < 4; ++a)
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
-        const int n = n0 + wn * 64 + b * 32 + 8 * rq + 4 * lh;
-        _Float16* yp = y + (size_t)tok * ldy + n;
+        const int n = n0 + wn * 128 + a * 32 + 8 * rq + 4 * lg;
+        if (n >= P.N) continue;
+        _Float16* yp = P.y + (size_t)tok * P.ldy + n;
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = acc[a][b][rq * 4 + r];
-        if (accumulate) {
+        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][rq * 4 + e];
+        if (P.accumulate) {
           const h4_t o = *(const h4_t*)yp;
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] += (float)o[r];
+          for (int e = 0; e < 4; ++e) v[e] += (float)o[e];
         }
-        h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+        const h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
         *(h4_t*)yp = o;
       }
   }
 }
 
-}  // namespace
-
-static int gemm_launch(const uint16_t* x, const uint16_t* w, const uint16_t* w2, uint16_t* y, int T,
-                       int K, int N, int accumulate, int ldy, void* stream) {
-  if (!x || !w || !y) return DZ_EINVAL;
-  if (T < 1 || K < 1 || N < 1 || K % TK || N % TN || ldy < N || ldy % 4) return DZ_ESHAPE;
-  if (((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)w2 & 15) || ((uintptr_t)y & 7)) return DZ_EALIGN;
-  const int total = ((T + TM - 1) / TM) * (N / TN);
-  const int grid = (total + 7) / 8 * 8;
-  hipLaunchKernelGGL(dz_gemm_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
-                     (const _Float16*)x, (const _Float16*)w, (const _Float16*)w2, (_Float16*)y, T, K, N,
-                     accumulate, ldy);
+int gemm_launch(GemmParams P, int ntiles_m, void* stream) {
+  if (!P.x || (!P.w && !P.w2) || !P.y) return DZ_EINVAL;
+  if (P.T < 1 || P.K < 1 || P.N < 1 || P.K % BK || P.N % 4 || P.ldy < P.N || P.ldy % 4 || ntiles_m < 1) return DZ_ESHAPE;
+  if (((uintptr_t)P.x & 15) || ((uintptr_t)P.w & 15) || ((uintptr_t)P.w2 & 15) || ((uintptr_t)P.y & 7) ||
+      (P.w2 && (P.w2_stride & 7)))
+    return DZ_EALIGN;
+  if ((unsigned long long)P.T * (unsigned)P.K * 2ull >= (1ull << 32) ||
+      (unsigned long long)P.N * (unsigned)P.K * 2ull >= (1ull << 32))
+    return DZ_ESHAPE;   // 32-bit row offsets inside one operand
+  P.tiles_m = ntiles_m;
+  P.tiles_n = (P.N + BN - 1) / BN;
+  const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
+  const int nsb = (sbm * sbn + 7) / 8 * 8;
+  const unsigned grid = (unsigned)nsb * GM * GN;
+  const size_t lds = 2 * 2 * SLAB;
+  static bool attr_done = false;
+  if (!attr_done) {
+    if (hipFuncSetAttribute((const void*)dz_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return DZ_ELAUNCH;
+    attr_done = true;
+  }
+  hipLaunchKernelGGL(dz_gemm_kernel, dim3(grid), dim3(256), lds, (hipStream_t)stream, P);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
+GemmParams base_params(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
+                       int accumulate, int ldy) {
+  GemmParams P{};
+  P.x = (const _Float16*)x; P.w = (const _Float16*)w; P.y = (_Float16*)y;
+  P.T = T; P.K = K; P.N = N; P.accumulate = accumulate; P.ldy = ldy;
+  return P;
+}
+
+}  // namespace
+
 extern "C" int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K, int N,
                            int accumulate, int ldy, void* stream) {
-  return gemm_launch(x, w, nullptr, y, T, K, N, accumulate, ldy, stream);
+  if (!w) return DZ_EINVAL;
+  return gemm_launch(base_params(x, w, y, T, K, N, accumulate, ldy), T < 1 ? 0 : (T + BM - 1) / BM, stream);
 }
 
 extern "C" int dz_gemm_f16_pair(const uint16_t* x, const uint16_t* w_a, const uint16_t* w_b, uint16_t* y,
                                 int T, int K, int N, int accumulate, int ldy, void* stream) {
-  if (!w_b) return DZ_EINVAL;
-  return gemm_launch(x, w_a, w_b, y, T, K, N, accumulate, ldy, stream);
+  if (!w_a || !w_b) return DZ_EINVAL;
+  // one group that spans all rows: the implicit 256-row blocks, all with second weight 0
+  GemmParams P = base_params(x, w_a, y, T, K, N, accumulate, ldy);
+  P.w2 = (const _Float16*)w_b;
+  return gemm_launch(P, T < 1 ? 0 : (T + BM - 1) / BM, stream);
+}
+
+extern "C" int dz_gemm_f16_grouped(const uint16_t* x, const uint16_t* w, const uint16_t* w2_stack,
+                                   long long w2_stride, const dz_gemm_tile* tiles, int ntiles, uint16_t* y,
+                                   int T, int K, int N, int accumulate, int ldy, void* stream) {
+  if (!tiles || ntiles < 1) return DZ_EINVAL;
+  GemmParams P = base_params(x, w, y, T, K, N, accumulate, ldy);
+  P.w2 = (const _Float16*)w2_stack; P.w2_stride = w2_stride; P.tiles = tiles;
+  return gemm_launch(P, ntiles, stream);
 }

@@ -1,5 +1,6 @@
-"""Prefill-sized calls (T > 128): per delta segment, dequantise the delta (dz_dequant, bit-exact)
-and run the dense matrix-core GEMM over base and delta together (dz_gemm_f16_pair).
+"""Prefill-sized calls (T > 128): sort the tokens by delta id, dequantise the deltas that are
+present (dz_dequant, bit-exact) and run one grouped matrix-core GEMM over base and delta together
+(dz_gemm_f16_grouped): every block of 256 tokens multiplies the base weight and its own delta.
 
 This is the strategy the reference's exllama backend switches to above 50 rows: reconstruct the
 weight, then a dense half-precision GEMM (serving/csrc/quantization/deltazip/exllama/cuda/
@@ -33,6 +34,9 @@ def gemm_f16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
     return out
 
 
+SCRATCH_LIMIT_BYTES = 4 << 30   # dequantised deltas held at once
+
+
 def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices,
                                *, bits: int, out: torch.Tensor, accumulate: bool) -> torch.Tensor:
     from .ops import segment
@@ -41,6 +45,7 @@ def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked,
     S = qweight_stacked.shape[0]
     G = scales_stacked[0].numel() // N
     group_size = -1 if G == 1 else K // G
+    lib = _lib.lib()
     perm, seg_off = segment(indices, S)
     off = seg_off.cpu().tolist()          # segment sizes decide the launches: one host sync
     perm64 = perm.long()
@@ -50,31 +55,37 @@ def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked,
     if not in_order and accumulate:
         ys.copy_(out.index_select(0, perm64))
     stream = torch.cuda.current_stream().cuda_stream
+
+    def blocks(lo, hi, group):
+        return [(r, min(r + 256, hi), group, 0) for r in range(lo, hi, 256)]
+
+    present = [d for d in range(S) if off[d + 2] > off[d + 1]]
+    per_chunk = max(1, SCRATCH_LIMIT_BYTES // (N * K * 2))
+    chunks = [present[i:i + per_chunk] for i in range(0, len(present), per_chunk)] or [[]]
     scratch = None
-    for s in range(S + 1):
-        lo, hi = off[s], off[s + 1]
-        if hi == lo:
-            continue
-        w2 = None
-        if s == 0:
-            if base_weight is None:
-                if not accumulate:
-                    ys[lo:hi].zero_()
-                continue
-            w = base_weight
-        else:
-            d = s - 1
-            if scratch is None:
-                scratch = torch.empty((N, K), dtype=torch.float16, device=x2.device)
-            rc = _lib.lib().dz_dequant(qweight_stacked[d].data_ptr(), meta_stacked[d].data_ptr(),
-                                       scales_stacked[d].data_ptr(), K, N, bits, group_size,
-                                       scratch.data_ptr(), stream)
-            _lib.check(rc, "dz_dequant")
+    for ci, chunk in enumerate(chunks):
+        tiles = []
+        if ci == 0 and off[1] > off[0]:               # tokens without a delta
             if base_weight is not None:
-                w, w2 = base_weight, scratch
-            else:
-                w = scratch
-        gemm_f16(xs[lo:hi], w, ys[lo:hi], accumulate, w2)
+                tiles += blocks(off[0], off[1], -1)
+            elif not accumulate:
+                ys[off[0]:off[1]].zero_()
+        if chunk and scratch is None:
+            scratch = torch.empty((min(per_chunk, len(present)), N, K), dtype=torch.float16, device=x2.device)
+        for j, d in enumerate(chunk):
+            rc = lib.dz_dequant(qweight_stacked[d].data_ptr(), meta_stacked[d].data_ptr(),
+                                scales_stacked[d].data_ptr(), K, N, bits, group_size,
+                                scratch[j].data_ptr(), stream)
+            _lib.check(rc, "dz_dequant")
+            tiles += blocks(off[d + 1], off[d + 2], j)
+        if not tiles:
+            continue
+        tt = torch.tensor(tiles, dtype=torch.int32, device=x2.device)
+        rc = lib.dz_gemm_f16_grouped(xs.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
+                                     scratch.data_ptr() if scratch is not None else None, N * K,
+                                     tt.data_ptr(), len(tiles), ys.data_ptr(), T, K, N,
+                                     1 if accumulate else 0, ys.stride(0), stream)
+        _lib.check(rc, "dz_gemm_f16_grouped")
     if not in_order:
         out.index_copy_(0, perm64, ys)
     return out

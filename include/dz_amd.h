@@ -111,6 +111,23 @@ int dz_gemm_f16(const uint16_t* x, const uint16_t* w, uint16_t* y, int T, int K,
 int dz_gemm_f16_pair(const uint16_t* x, const uint16_t* w_a, const uint16_t* w_b, uint16_t* y,
                      int T, int K, int N, int accumulate, int ldy, void* stream);
 
+/* One block of consecutive rows (tokens) of a grouped GEMM: rows [row_lo, row_hi), at most 256 of
+ * them, all using second weight `group` (-1: none). */
+typedef struct dz_gemm_tile {
+  int row_lo, row_hi, group, reserved;
+} dz_gemm_tile;
+
+/* Grouped form of dz_gemm_f16_pair for a batch sorted by delta id: y[t] (+)= x[t] @ w^T +
+ * x[t] @ w2_stack[group(t)]^T, where `tiles` (device memory, ntiles entries) cuts the rows into
+ * blocks that do not straddle groups and w2_stack + group * w2_stride (elements) is the [N, K]
+ * second weight of a group.  w may be NULL (second product only).  Rows not covered by a tile
+ * are not written.  This is the batched
+ * form of the per-delta loop of the reference's dense fallbacks (for id in unique(indices):
+ * F.linear(x[indices == id], W[id]); serving/vllm/delta/deltazip_marlin.py:44-53). */
+int dz_gemm_f16_grouped(const uint16_t* x, const uint16_t* w, const uint16_t* w2_stack,
+                        long long w2_stride, const dz_gemm_tile* tiles, int ntiles, uint16_t* y,
+                        int T, int K, int N, int accumulate, int ldy, void* stream);
+
 /* Tuning hook used by the benchmark: override the split of K across workgroups of the fused
  * kernel (0 = automatic). */
 void dz_set_ksplit(int nsplit);
