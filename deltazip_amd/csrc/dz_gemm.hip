@@ -85,17 +85,25 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
     const int lc = (lane & 7) ^ ((R >> 1) & 7);
     goff[i] = rowoff * Kb + (unsigned)lc * 16u;
   }
+  // (buffer form of the LDS-direct load: scalar descriptor + 32-bit lane offset + scalar slab
+  // offset, so no 64-bit per-lane address is ever built or kept)
+  const __amdgpu_buffer_rsrc_t rw =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.w ? P.w : w2), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rw2 =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(w2 ? w2 : P.w), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rx =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.x), 0, 0x7fffffff, 0x00020000);
   auto issue = [&](int s, int buf) {
     const bool second = s >= nslab1;
-    const char* wsrc = (const char*)(second ? w2 : P.w) + (size_t)(second ? s - nslab1 : s) * (BK * 2);
-    const char* xsrc = (const char*)P.x + (size_t)(second ? s - nslab1 : s) * (BK * 2);
+    const int soff = (second ? s - nslab1 : s) * (BK * 2);
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int rq = wave * 16 + i, sub = rq & 31;
-      const char* src = (rq < 32 ? wsrc : xsrc) + goff[i];
       unsigned char* dst = smem + buf * (2 * SLAB) + (rq < 32 ? 0 : SLAB) + sub * 1024;
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                       (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+      __attribute__((address_space(3))) void* d3 = (__attribute__((address_space(3))) void*)dst;
+      if (rq >= 32) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, d3, 16, (int)goff[i], soff, 0, 0);
+      else if (second) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw2, d3, 16, (int)goff[i], soff, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, d3, 16, (int)goff[i], soff, 0, 0);
     }
   };
 
@@ -139,7 +147,12 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
     const int tok = row_lo + wm * 128 + b * 32 + li;
     if (tok >= row_hi) continue;
 #pragma unroll
-    for (int a = 0; a < 4; ++a)
+    for (int a = 0; a < 4; ++a) {
+      // The accumulators live in the accumulation registers; pinning each block there until its
+      // turn keeps the compiler from moving all 256 values to ordinary registers at once (which
+      // would push the loop's own values out to scratch memory).
+      f16_t blk = acc[a][b];
+      asm volatile("" : "+a"(blk));
 #pragma unroll
       for (int rq = 0; rq < 4; ++rq) {
         const int n = n0 + wn * 128 + a * 32 + 8 * rq + 4 * lg;
@@ -147,7 +160,7 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
         _Float16* yp = P.y + (size_t)tok * P.ldy + n;
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = acc[a][b][rq * 4 + e];
+        for (int e = 0; e < 4; ++e) v[e] = blk[rq * 4 + e];
         if (P.accumulate) {
           const h4_t o = *(const h4_t*)yp;
 #pragma unroll
@@ -156,6 +169,8 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
         const h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
         *(h4_t*)yp = o;
       }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // one token block at a time: the rest stays in the accumulators
   }
 }
 
