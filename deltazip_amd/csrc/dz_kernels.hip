@@ -96,13 +96,16 @@ __global__ __launch_bounds__(64) void dz_dequant_kernel(const uint32_t* __restri
 __global__ __launch_bounds__(1024) void dz_segment_kernel(const long long* __restrict__ idx, int T,
                                                           int S, int* __restrict__ perm,
                                                           int* __restrict__ seg_off) {
-  extern __shared__ int sm[];  // hist[S+2], running[S+1], keys[1024]
+  // hist[S+2] (exclusive offsets after the scan), running[S+1] (tokens of a key placed by earlier
+  // chunks), cnt[16][S+1] (tokens of a key per wavefront of the current chunk)
+  extern __shared__ int sm[];
   int* hist = sm;
   int* running = sm + (S + 2);
-  int* keys = running + (S + 1);
-  const int tid = threadIdx.x;
+  int* cnt = running + (S + 1);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int nk = S + 1;
   for (int s = tid; s < S + 2; s += 1024) hist[s] = 0;
-  for (int s = tid; s < S + 1; s += 1024) running[s] = 0;
+  for (int s = tid; s < nk; s += 1024) running[s] = 0;
   __syncthreads();
   for (int t = tid; t < T; t += 1024) {
     long long id = idx[t];
@@ -115,22 +118,38 @@ __global__ __launch_bounds__(1024) void dz_segment_kernel(const long long* __res
   }
   __syncthreads();
   for (int s = tid; s < S + 2; s += 1024) seg_off[s] = hist[s];
+  // chunks of 1024 tokens in order; inside a chunk a token's place among equal keys is
+  // (tokens of that key in earlier wavefronts) + (in lower lanes of its own wavefront)
   for (int base = 0; base < T; base += 1024) {
+    for (int c = tid; c < 16 * nk; c += 1024) cnt[c] = 0;
+    __syncthreads();
     const int t = base + tid;
     int key = -1;
     if (t < T) {
       long long id = idx[t];
       key = (id < 0 || id >= S) ? 0 : (int)id + 1;
     }
-    keys[tid] = key;
-    __syncthreads();
-    if (t < T) {
-      int r = 0;
-      for (int u = 0; u < tid; ++u) r += (keys[u] == key);
-      perm[hist[key] + running[key] + r] = t;
+    int rank = 0;
+    unsigned long long todo = __builtin_amdgcn_ballot_w64(key >= 0);
+    while (todo) {
+      const int k = __builtin_amdgcn_readlane(key, __builtin_ctzll(todo));
+      const unsigned long long m = __builtin_amdgcn_ballot_w64(key == k);
+      if (key == k) rank = __builtin_popcountll(m & ((1ull << lane) - 1ull));
+      if (lane == 0) cnt[wave * nk + k] = __builtin_popcountll(m);
+      todo &= ~m;
     }
     __syncthreads();
-    if (t < T) atomicAdd(&running[key], 1);
+    if (t < T) {
+      int before = 0;
+      for (int w = 0; w < wave; ++w) before += cnt[w * nk + key];
+      perm[hist[key] + running[key] + before + rank] = t;
+    }
+    __syncthreads();
+    for (int k = tid; k < nk; k += 1024) {
+      int tot = 0;
+      for (int w = 0; w < 16; ++w) tot += cnt[w * nk + k];
+      running[k] += tot;
+    }
     __syncthreads();
   }
 }
@@ -602,8 +621,8 @@ int dz_merge(const uint16_t* w_base, const void* codes, const void* meta, const 
 
 int dz_segment(const int64_t* indices, int T, int S, int32_t* perm, int32_t* seg_off, void* stream) {
   if (!indices || !perm || !seg_off) return DZ_EINVAL;
-  if (T < 1 || S < 0 || S > 8192) return DZ_ESHAPE;
-  const size_t lds = (size_t)((S + 2) + (S + 1) + 1024) * 4;
+  if (T < 1 || S < 0 || S > DZ_MAX_SLOTS_SEGMENT) return DZ_ESHAPE;
+  const size_t lds = (size_t)((S + 2) + (S + 1) + 16 * (S + 1)) * 4;   // < 64 KiB
   hipLaunchKernelGGL(dz_segment_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream,
                      (const long long*)indices, T, S, perm, seg_off);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;

@@ -41,6 +41,7 @@ extern "C" {
 #define DZ_EALIGN      -10   /* pointer not aligned as required                            */
 
 #define DZ_MAX_TOKENS_FUSED 128   /* largest T the fused decode kernel takes in one launch   */
+#define DZ_MAX_SLOTS_SEGMENT 768   /* largest S dz_segment takes (its tables live in LDS)      */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int dz_version(void);
@@ -75,7 +76,7 @@ int dz_merge(const uint16_t* w_base, const void* codes, const void* meta, const 
 
 /* Group tokens by delta id: perm[T] lists token indices sorted by id (stable; id -1 first),
  * seg_off[S + 2] are the offsets of the segments for id = -1, 0, ..., S-1 in perm.
- * Ids outside [-1, S) are treated as -1.  (The reference's scheduler sorts the batch by delta
+ * Ids outside [-1, S) are treated as -1; S <= DZ_MAX_SLOTS_SEGMENT.  (The reference's scheduler sorts the batch by delta
  * id, serving/vllm/core/scheduler.py:101-104; this makes the op independent of that.) */
 int dz_segment(const int64_t* indices, int T, int S, int32_t* perm, int32_t* seg_off, void* stream);
 
