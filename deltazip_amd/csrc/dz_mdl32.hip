@@ -70,6 +70,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
       boff[tt][c] = (tt * 16 + jj) * (DZ_KBLOCK * 2) + ((((c << 2) | ga) ^ jj) << 4);
 
   u4_t a[2][4][2];  // base tile: [row fragment][step][half]
+  int prow = 0;     // row of x / y / idx that holds this launch's token `lane`
 
   // Activations slice of k-block kb -> LDS, rows in token order; rows >= T repeat row T-1 (they
   // only feed output columns that are never stored).  Addresses are a wavefront-uniform base plus
@@ -79,7 +80,8 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
       const int t = min(2 * i + (lane_r >> 5), P.T - 1), c = lane_r & 31;
-      const unsigned off = (unsigned)t * Kb + (unsigned)((c ^ (t & 15)) << 4);
+      const int row = __builtin_amdgcn_ds_bpermute(t << 2, prow);
+      const unsigned off = (unsigned)row * Kb + (unsigned)((c ^ (t & 15)) << 4);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
                                        (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
                                        16, 0, 0);
@@ -108,7 +110,10 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   // The ids are requested before anything else and nothing more is requested until they are in:
   // a request queued behind this kernel's own flood of weight loads takes several microseconds.
   long long id = -1;
-  if (lane < P.T) id = P.idx[lane];
+  if (lane < P.T) {
+    prow = P.perm ? P.perm[P.tok0 + lane] : P.tok0 + lane;
+    id = P.idx[prow];
+  }
   __builtin_amdgcn_sched_barrier(0);
 
   for (int r = 0; r < nrounds; ++r) {
@@ -304,9 +309,12 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   }
 
   // ---- reduce over the 4 wavefronts (LDS), then over the k-chunks of other workgroups
+  int yrow[TT];   // output row of column tt*16 + jj
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) yrow[tt] = __builtin_amdgcn_ds_bpermute((tt * 16 + jj) << 2, prow);
   auto final_store = [&](int s, int tt, f4_t v) {
     if (tt * 16 + jj < P.T) {
-      _Float16* yp = P.y + (size_t)(tt * 16 + jj) * P.ldy + n0 + 16 * s + 4 * ga;
+      _Float16* yp = P.y + (size_t)yrow[tt] * P.ldy + n0 + 16 * s + 4 * ga;
       if (P.accumulate) {
         const h4_t o = *(const h4_t*)yp;
         v += (f4_t){(float)o[0], (float)o[1], (float)o[2], (float)o[3]};
