@@ -87,6 +87,7 @@ struct MdlParams {
   unsigned* status;
   const int* perm;   // token order (rows of x / y / idx) or nullptr: rows tok0, tok0 + 1, ...
   int tok0;          // first position of this launch in that order; T counts from there
+  int nchunk;        // chunks of 32 tokens in this launch (1..4)
   long long codes_slot_u4, meta_slot_u4, scales_slot;
   int T, K, N, S, G, gs;
   int accumulate, ldy, nsplit, cb;

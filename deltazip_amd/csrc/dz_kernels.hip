@@ -165,7 +165,7 @@ inline int check_group(int K, int group_size, int* gs_out) {
 }
 
 constexpr size_t WS_HEADER = 256;  // status word
-inline size_t ws_counter_bytes(int N) { return (((size_t)(N / DZ_NPAIR + 8) * 4) + 255) / 256 * 256; }
+inline size_t ws_counter_bytes(int N) { return (((size_t)(N / DZ_NPAIR + 8) * 4 * 4) + 255) / 256 * 256; }   // 4 chunks
 constexpr int MAX_KSPLIT = 16;
 constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // segment offsets + token order
 
@@ -294,17 +294,12 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
   P.perm = nullptr;
   P.tok0 = 0;
   if (T <= 32) return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
-  // 33..128 tokens: order the tokens by delta id on the device (no host round trip), then one
-  // launch per 32 tokens of that order, so that a chunk meets as few deltas as possible
+  // 33..128 tokens: order the tokens by delta id on the device (no host round trip), so that each
+  // chunk of 32 meets as few deltas as possible; one launch carries all chunks
   if (S > DZ_MAX_SLOTS_SEGMENT) return DZ_ESHAPE;
   if ((rc = dz_segment(indices, T, S, perm, seg_off, stream))) return rc;
   P.perm = perm;
-  for (int t0 = 0; t0 < T; t0 += 32) {
-    P.tok0 = t0;
-    P.T = T - t0 < 32 ? T - t0 : 32;
-    if ((rc = dz_launch_mdl32(P, bits, pre, st, g_ksplit_override))) return rc;
-  }
-  return DZ_OK;
+  return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
 }
 
 }  // extern "C"

@@ -41,9 +41,15 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 
   // workgroup -> (n-pair, k-chunk); the chunks of one n-pair are dealt to one XCD so that their
   // partial sums can meet in that XCD's L2
+  // A launch may carry up to 4 chunks of 32 tokens (33..128 tokens, ordered by delta id): the
+  // workgroups of the chunks of one (n-pair, k-chunk) follow each other on the same XCD, so the
+  // base tile they all read comes from HBM once.
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-  const int np = (q / P.nsplit) * 8 + xcd, kc = q % P.nsplit;
+  const int per = P.nsplit * P.nchunk, rem = q % per;
+  const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
   if (np >= P.NP) return;
+  const int tok0 = P.tok0 + 32 * ch;
+  const int Tc = min(32, P.T - 32 * ch);   // tokens of this chunk
   const int n0 = np * DZ_NPAIR;
   const int kb_lo = kc * P.cb, kb_hi = min(P.NKB, kb_lo + P.cb);
   const int nrounds = (kb_hi - kb_lo + WK32 - 1) / WK32;
@@ -79,7 +85,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
 #pragma unroll
     for (int i = 0; i < NX; ++i) {
-      const int t = min(2 * i + (lane_r >> 5), P.T - 1), c = lane_r & 31;
+      const int t = min(2 * i + (lane_r >> 5), Tc - 1), c = lane_r & 31;
       const int row = __builtin_amdgcn_ds_bpermute(t << 2, prow);
       const unsigned off = (unsigned)row * Kb + (unsigned)((c ^ (t & 15)) << 4);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
@@ -110,8 +116,8 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   // The ids are requested before anything else and nothing more is requested until they are in:
   // a request queued behind this kernel's own flood of weight loads takes several microseconds.
   long long id = -1;
-  if (lane < P.T) {
-    prow = P.perm ? P.perm[P.tok0 + lane] : P.tok0 + lane;
+  if (lane < Tc) {
+    prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
     id = P.idx[prow];
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -126,9 +132,9 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 
     if (r == 0) {
       // nothing is requested before the ids are in (see above)
-      if (lane < P.T) {
+      if (lane < Tc) {
         key = (id < 0 || id >= P.S) ? 0 : (int)id + 1;
-        if ((id < -1 || id >= P.S) && blockIdx.x == 0 && wave == 0) atomicOr(P.status, 1u);
+        if ((id < -1 || id >= P.S) && np == 0 && kc == 0 && wave == 0) atomicOr(P.status, 1u);
       }
       // tokens that carry a delta; lanes >= T never match
       mdelta = __builtin_amdgcn_ballot_w64(key != 0 && key != 0x7fffffff);
@@ -313,7 +319,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) yrow[tt] = __builtin_amdgcn_ds_bpermute((tt * 16 + jj) << 2, prow);
   auto final_store = [&](int s, int tt, f4_t v) {
-    if (tt * 16 + jj < P.T) {
+    if (tt * 16 + jj < Tc) {
       _Float16* yp = P.y + (size_t)yrow[tt] * P.ldy + n0 + 16 * s + 4 * ga;
       if (P.accumulate) {
         const h4_t o = *(const h4_t*)yp;
@@ -327,7 +333,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   // written and read with agent-scope accesses (write-through / cache-bypassing), so that no
   // whole-cache write-back or invalidate is needed to pass them between XCDs.
   auto part_ptr = [&](int kc2, int item) -> float* {
-    return P.partials + (((size_t)kc2 * P.NP + np) * (2 * TT) + item) * 256 + lane;
+    return P.partials + (((size_t)(ch * P.nsplit + kc2) * P.NP + np) * (2 * TT) + item) * 256 + lane;
   };
 
   __syncthreads();  // every wavefront is done with its activations: LDS becomes the buffer
@@ -366,7 +372,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   }
   __syncthreads();
   if (tid == 0) {
-    const unsigned old = atomicAdd(P.counters + np, 1u);
+    const unsigned old = atomicAdd(P.counters + ch * P.NP + np, 1u);
     s_last = (old == (unsigned)(P.nsplit - 1));
   }
   __syncthreads();
@@ -382,7 +388,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
       }
       store_item(tot);
     }
-    if (tid == 0) P.counters[np] = 0u;
+    if (tid == 0) P.counters[ch * P.NP + np] = 0u;
   }
   DZ_TS(9);
 }
@@ -394,14 +400,14 @@ int launch32(MdlParams P, bool pre, hipStream_t st, int ksplit_override) {
   if (nsplit <= 0) {
     nsplit = 1;
     const int max_split = (P.NKB + WK32 - 1) / WK32;  // at least one round of 4 k-blocks each
-    while (nsplit < max_split && (long long)P.NP * nsplit < 512) ++nsplit;
+    while (nsplit < max_split && (long long)P.NP * nsplit * P.nchunk < 512) ++nsplit;
   }
-  if (nsplit > 16) nsplit = 16;
+  if (nsplit > 16 / P.nchunk) nsplit = 16 / P.nchunk;   // the workspace holds 16 sets of partial sums
   if (nsplit > P.NKB) nsplit = P.NKB;
   P.cb = (P.NKB + nsplit - 1) / nsplit;
   P.cb = (P.cb + WK32 - 1) / WK32 * WK32;  // whole rounds
   P.nsplit = (P.NKB + P.cb - 1) / P.cb;
-  const int grid = (P.NP + 7) / 8 * 8 * P.nsplit;
+  const int grid = (P.NP + 7) / 8 * 8 * P.nsplit * P.nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
   static bool attr_done[4] = {false, false, false, false};
   const bool has_base = P.wb != nullptr;
@@ -424,7 +430,10 @@ int launch32(MdlParams P, bool pre, hipStream_t st, int ksplit_override) {
 }  // namespace
 
 // Launch of the T <= 32 kernel; called by dz_multi_delta_linear.
-int dz_launch_mdl32(const MdlParams& P, int bits, bool pre, hipStream_t st, int ksplit_override) {
+int dz_launch_mdl32(const MdlParams& P0, int bits, bool pre, hipStream_t st, int ksplit_override) {
+  MdlParams P = P0;
+  P.nchunk = (P.T + 31) / 32;
+  if (P.nchunk < 1 || P.nchunk > 4) return DZ_ESHAPE;
   if (bits == 2) return P.T <= 16 ? launch32<2, 1>(P, pre, st, ksplit_override) : launch32<2, 2>(P, pre, st, ksplit_override);
   return P.T <= 16 ? launch32<4, 1>(P, pre, st, ksplit_override) : launch32<4, 2>(P, pre, st, ksplit_override);
 }
