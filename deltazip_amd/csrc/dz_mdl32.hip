@@ -379,12 +379,21 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   DZ_TS(8);
   if (s_last) {
     if (has_item) {
+      // eight K-slices per turn: all their loads are in flight together (one memory round trip
+      // instead of eight), the additions stay in slice order
       f4_t tot = {0.f, 0.f, 0.f, 0.f};
-      for (int k2 = 0; k2 < P.nsplit; ++k2) {
-        const float* pp = part_ptr(k2, wave);
+      for (int k0 = 0; k0 < P.nsplit; k0 += 8) {
+        f4_t v[8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e)
-          tot[e] += __hip_atomic_load(pp + 64 * e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int u = 0; u < 8; ++u) {
+          const float* pp = part_ptr(min(k0 + u, P.nsplit - 1), wave);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            v[u][e] = __hip_atomic_load(pp + 64 * e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (k0 + u < P.nsplit) tot += v[u];
       }
       store_item(tot);
     }
