@@ -222,3 +222,64 @@ def test_prefill_sized_call(dev, kind):
     y = run_layer(p).cpu().numpy()
     ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
     assert o.rel_err(y, ref) <= TOL
+
+
+def test_gemm_grouped(dev):
+    """Grouped GEMM through the C ABI: ragged row blocks, a block without second weight, rows that no
+    block covers (left untouched), an N that is not a multiple of the 256-wide tile, and the
+    second-product-only form (w = NULL)."""
+    from deltazip_amd import _lib
+    L = _lib.lib()
+    torch.manual_seed(1)
+    T, K, N, G = 700, 512, 352, 3
+    x = torch.randn(T, K, device=dev).half()
+    w = (torch.randn(N, K, device=dev) * 0.05).half()
+    w2 = (torch.randn(G, N, K, device=dev) * 0.05).half()
+    blocks = [(0, 100, -1), (100, 356, 2), (356, 390, 2), (390, 391, 0), (400, 656, 1), (656, 700, 1)]
+    tiles = torch.tensor([(lo, hi, g, 0) for lo, hi, g in blocks], dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    for with_base in (True, False):
+        y = torch.full((T, N), 7.0, dtype=torch.float16, device=dev)
+        rc = L.dz_gemm_f16_grouped(x.data_ptr(), w.data_ptr() if with_base else None, w2.data_ptr(), N * K,
+                                   tiles.data_ptr(), len(blocks), y.data_ptr(), T, K, N, 0, N, st)
+        assert rc == 0
+        torch.cuda.synchronize()
+        ref = torch.full((T, N), 7.0, dtype=torch.float32, device=dev)
+        for lo, hi, g in blocks:
+            r = x[lo:hi].float() @ w.float().t() if with_base else None
+            if g >= 0:
+                d = x[lo:hi].float() @ w2[g].float().t()
+                r = d if r is None else r + d
+            if r is not None:
+                ref[lo:hi] = r
+        assert o.rel_err(y.float().cpu().numpy(), ref.cpu().numpy()) <= 2e-3
+        assert torch.equal(y[391:400], torch.full((9, N), 7.0, dtype=torch.float16, device=dev))
+    # argument checks happen before the launch
+    assert L.dz_gemm_f16_grouped(x.data_ptr(), w.data_ptr(), w2.data_ptr(), N * K, None, 1, y.data_ptr(),
+                                 T, K, N, 0, N, st) != 0
+    assert L.dz_gemm_f16_grouped(x.data_ptr(), w.data_ptr(), w2.data_ptr(), N * K, tiles.data_ptr(), 1,
+                                 y.data_ptr(), T, K + 8, N, 0, N, st) != 0
+
+
+def test_segment_limits(dev):
+    ids = torch.zeros(10, dtype=torch.int64, device=dev)
+    perm = torch.empty(10, dtype=torch.int32, device=dev)
+    from deltazip_amd import _lib
+    off = torch.empty(2000, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    assert _lib.lib().dz_segment(ids.data_ptr(), 10, 768, perm.data_ptr(), off.data_ptr(), st) == 0
+    assert _lib.lib().dz_segment(ids.data_ptr(), 10, 769, perm.data_ptr(), off.data_ptr(), st) != 0
+    torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("t", [33, 64, 97, 128])
+def test_unsorted_batches_above_32_tokens(dev, t):
+    """33..128 tokens in arbitrary order with many deltas: the device-side ordering must bring every
+    token back to its own output row."""
+    p = make_problem(96, 768, 4, 128, 20, t, "uniform", 4242 + t, dev)
+    p["ids_np"][::7] = -1
+    p["ids"] = torch.from_numpy(p["ids_np"]).to(dev)
+    y = run_layer(p).cpu().numpy()
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    assert o.rel_err(y, ref) <= TOL
+    assert ops.workspace_status() == 0
