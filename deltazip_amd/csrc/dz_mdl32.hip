@@ -146,6 +146,10 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     // of their first token, G at a time; `pop` takes the next one and returns the output columns
     // (tokens) that belong to it.  The loader runs two batches ahead of the consumer.
     Frag<BITS> ring[2][G];
+    // PRE: scales of the batch, one fp16 per lane and register: lane l holds row n0 + l%32 of the
+    // k-block's scale group l/32 (register 0) and l/32 + 2 (register 1); a step's scale reaches the
+    // lane that multiplies with it through a cross-lane move, not through memory
+    unsigned rsc[2][G][2];
     unsigned long long ld_m = mdelta, use_m = mdelta;
     auto pop = [&](unsigned long long& m, int& kd, unsigned long long& cols) {
       const int l = __builtin_ctzll(m);
@@ -155,7 +159,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     };
     // Always G requests, so that the number of loads in flight is known at compile time and the
     // waits in front of each use can be exact: a slot without a delta re-reads 16 bytes.
-    auto load_batch = [&](Frag<BITS> (&slot)[G]) {
+    auto load_batch = [&](Frag<BITS> (&slot)[G], unsigned (&rs)[G][2]) {
 #pragma unroll
       for (int g = 0; g < G; ++g) {
         int kd = 1;
@@ -163,13 +167,20 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
         const bool real = ld_m != 0;
         if (real) pop(ld_m, kd, cols);
         slot[g] = load_frag<BITS>(P, kd - 1, np, kb, real ? lane_r : 0);
+        if (PRE) {
+          const int ls = real ? lane_r : 0;
+          const int gb0 = (kb * DZ_KBLOCK) / P.gs + (ls >> 5);
+          const _Float16* sb = P.scales + (size_t)(kd - 1) * P.scales_slot + n0 + (ls & 31);
+          rs[g][0] = *(const unsigned short*)(sb + (size_t)min(gb0, P.G - 1) * P.N);
+          rs[g][1] = *(const unsigned short*)(sb + (size_t)min(gb0 + 2, P.G - 1) * P.N);
+        }
       }
     };
 
     // ---- issue order: activations (L2 -> LDS), packed deltas of two batches, base tile
     issue_x(kb, lane_r);
-    load_batch(ring[0]);
-    load_batch(ring[1]);
+    load_batch(ring[0], rsc[0]);
+    load_batch(ring[1], rsc[1]);
     __builtin_amdgcn_sched_barrier(0);
     if (HAS_BASE) issue_base(kb, lane_r);
     __builtin_amdgcn_sched_barrier(0);
@@ -195,7 +206,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     };
     // one batch: for every column tile that holds tokens of these deltas, one pass over the four
     // steps in which each operand read feeds all deltas of the batch
-    auto consume = [&](Frag<BITS> (&slot)[G]) {
+    auto consume = [&](Frag<BITS> (&slot)[G], unsigned (&rs)[G][2]) {
       int kd[G];
       unsigned long long cols[G];
       unsigned long long any = 0;
@@ -232,11 +243,15 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
                 A1 = unpack4(slot[g].code[(BITS == 2) ? 0 : (j >> 1)][2 * (j & 1) + 1], MAGIC);
               }
               if (PRE) {
-                // the lane's operand row is n0 + 16*s + jj; one scale per (row, K-group)
-                const _Float16* sp = P.scales + (size_t)(kd[g] - 1) * P.scales_slot + n0 + jj +
-                                     (size_t)((kb * DZ_KBLOCK + 64 * j) / P.gs) * P.N;
-                A0 *= sp[0];
-                A1 *= sp[16];
+                // the lane's operand rows are n0 + jj and n0 + 16 + jj; one scale per (row, K-group)
+                const int gk = (kb * DZ_KBLOCK + 64 * j) / P.gs - (kb * DZ_KBLOCK) / P.gs;   // 0..3
+                const unsigned pick = 0u - (unsigned)((gk >> 1) & 1);   // all ones: groups 2, 3
+                const int v = (int)((rs[g][1] & pick) | (rs[g][0] & ~pick));
+                const int src = (jj + ((gk & 1) << 5)) << 2;
+                const unsigned short s0 = (unsigned short)__builtin_amdgcn_ds_bpermute(src, v);
+                const unsigned short s1 = (unsigned short)__builtin_amdgcn_ds_bpermute(src + 64, v);
+                A0 *= __builtin_bit_cast(_Float16, s0);
+                A1 *= __builtin_bit_cast(_Float16, s1);
               }
               const int mw = (int)slot[g].meta[j];
               t0[g] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B, t0[g], mw, 0, 0);
@@ -260,10 +275,10 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     };
 
     // first two batches in straight-line code; their data arrives before the base tile does
-    consume(ring[0]);
-    if (ld_m) load_batch(ring[0]);
-    consume(ring[1]);
-    if (ld_m) load_batch(ring[1]);
+    consume(ring[0], rsc[0]);
+    if (ld_m) load_batch(ring[0], rsc[0]);
+    consume(ring[1], rsc[1]);
+    if (ld_m) load_batch(ring[1], rsc[1]);
     // ---- base: dense matrix-core product over all token tiles
     if (HAS_BASE) {
 #pragma unroll
@@ -284,11 +299,11 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
     }
     // more than 2*G deltas: keep going, two batches per turn
     while (use_m) {
-      consume(ring[0]);
-      if (ld_m) load_batch(ring[0]);
+      consume(ring[0], rsc[0]);
+      if (ld_m) load_batch(ring[0], rsc[0]);
       if (use_m) {
-        consume(ring[1]);
-        if (ld_m) load_batch(ring[1]);
+        consume(ring[1], rsc[1]);
+        if (ld_m) load_batch(ring[1], rsc[1]);
       }
     }
     // Every load of this round has been consumed by now; saying so keeps the waits of the next
