@@ -268,7 +268,7 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
-                    "kernel": "dz_mdl32_kernel" if T <= 32 else "dz_mdl_kernel",
+                    "kernel": "dz_mdl32_kernel",
                     "algorithmic_bytes_per_launch": step_bytes // len(shapes),
                     "avg_launch_us": round(avg_launch_s * 1e6, 2)}
     else:

@@ -5,10 +5,12 @@
 Python keeps the reference's operator and layer API; all arithmetic runs in hand-written HIP
 kernels for gfx950 behind the C ABI declared in include/dz_amd.h.  There is no CPU fallback.
 """
+from .checkpoint import CompressionConfig, DeltaLayerWeights, DeltaModel, convert_model
 from .config import DeltaConfig
 from .layers import (BaseLayerWithDelta, ColumnParallelLinearWithDelta, DeltaMapping,
                      MergedColumnParallelLinearWithDelta, MergedQKVParallelLinearWithDelta,
                      RowParallelLinearWithDelta, convert_mapping, from_layer)
+from .manager import DeltaModelManager, LRUCacheDeltaModelManager, create_delta_manager
 from .ops import (add_delta, add_delta_slice, apply_delta, dequant, merge, multi_delta_linear,
                   native_sizes, repack_gptq_to_native, segment, stacked_shapes)
 from .quant_linear import QuantLinear
@@ -18,5 +20,7 @@ __all__ = [
     "MergedColumnParallelLinearWithDelta", "MergedQKVParallelLinearWithDelta",
     "RowParallelLinearWithDelta", "convert_mapping", "from_layer", "add_delta", "add_delta_slice",
     "apply_delta", "dequant", "merge", "multi_delta_linear", "native_sizes",
-    "repack_gptq_to_native", "segment", "stacked_shapes", "QuantLinear",
+    "repack_gptq_to_native", "segment", "stacked_shapes", "QuantLinear", "CompressionConfig",
+    "DeltaLayerWeights", "DeltaModel", "convert_model", "DeltaModelManager", "LRUCacheDeltaModelManager",
+    "create_delta_manager",
 ]

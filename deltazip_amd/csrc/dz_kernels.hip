@@ -153,6 +153,52 @@ __global__ __launch_bounds__(1024) void dz_segment_kernel(const long long* __res
 }
 
 // ---------------------------------------------------------------------------------------------
+// delta id -> slot index for every token and every sampled row (the manager's index tensors).
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dz_map_ids_kernel(const long long* __restrict__ token_ids, int T,
+                                                         const long long* __restrict__ prompt_ids, int P,
+                                                         const long long* __restrict__ slot_ids, int S,
+                                                         long long pad_slot, long long vocab,
+                                                         long long extra_vocab,
+                                                         long long* __restrict__ base_indices,
+                                                         long long* __restrict__ sampler_indices,
+                                                         long long* __restrict__ sampler_padded,
+                                                         long long* __restrict__ emb_indices, int ld_emb,
+                                                         int* __restrict__ n_missing) {
+  extern __shared__ long long table[];
+  for (int s = threadIdx.x; s < S; s += 256) table[s] = slot_ids[s];
+  __syncthreads();
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  auto find = [&](long long id, bool& missing) -> long long {
+    missing = false;
+    if (id <= 0) return -1;
+    for (int s = 0; s < S; ++s)
+      if (table[s] == id) return s;
+    missing = true;
+    return -1;
+  };
+  bool miss;
+  if (i < T) {
+    const long long id = token_ids[i];
+    const long long slot = find(id, miss);
+    if (miss && n_missing) atomicAdd(n_missing, 1);
+    base_indices[i] = slot;
+    if (emb_indices) {
+      const long long e = id > 0 ? slot : 0;
+      long long e0 = e * extra_vocab, e1 = e * (vocab + extra_vocab);
+      emb_indices[i] = e0 == -1 ? pad_slot : e0;
+      emb_indices[ld_emb + i] = e1 == -1 ? pad_slot : e1;
+    }
+  }
+  if (i < P && sampler_indices) {
+    const long long slot = find(prompt_ids[i], miss);
+    if (miss && n_missing) atomicAdd(n_missing, 1);
+    sampler_indices[i] = slot;
+    if (sampler_padded) sampler_padded[i] = (long long)i + (slot == -1 ? pad_slot : slot) * (long long)P;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 int g_ksplit_override = 0;
@@ -242,6 +288,23 @@ int dz_segment(const int64_t* indices, int T, int S, int32_t* perm, int32_t* seg
   const size_t lds = (size_t)((S + 2) + (S + 1) + 16 * (S + 1)) * 4;   // < 64 KiB
   hipLaunchKernelGGL(dz_segment_kernel, dim3(1), dim3(1024), lds, (hipStream_t)stream,
                      (const long long*)indices, T, S, perm, seg_off);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+int dz_map_ids(const int64_t* token_ids, int T, const int64_t* prompt_ids, int P,
+               const int64_t* slot_ids, int S, int max_deltas, int vocab_size, int extra_vocab_size,
+               int64_t* base_indices, int64_t* sampler_indices, int64_t* sampler_indices_padded,
+               int64_t* embeddings_indices, int ld_emb, int32_t* n_missing, void* stream) {
+  if (!token_ids || !slot_ids || !base_indices) return DZ_EINVAL;
+  if (P > 0 && (!prompt_ids || !sampler_indices)) return DZ_EINVAL;
+  if (T < 1 || P < 0 || S < 1 || S > DZ_MAX_SLOTS_MAP || max_deltas < 1) return DZ_ESHAPE;
+  if (embeddings_indices && ld_emb < T) return DZ_ESHAPE;
+  const int n = T > P ? T : P;
+  hipLaunchKernelGGL(dz_map_ids_kernel, dim3((n + 255) / 256), dim3(256), (size_t)S * 8,
+                     (hipStream_t)stream, (const long long*)token_ids, T, (const long long*)prompt_ids,
+                     P, (const long long*)slot_ids, S, (long long)max_deltas - 1, (long long)vocab_size,
+                     (long long)extra_vocab_size, (long long*)base_indices, (long long*)sampler_indices,
+                     (long long*)sampler_indices_padded, (long long*)embeddings_indices, ld_emb, n_missing);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 

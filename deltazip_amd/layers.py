@@ -141,6 +141,8 @@ class LinearWithDelta(BaseLayerWithDelta):
     def can_replace_layer(cls, source_layer: nn.Module, delta_config: DeltaConfig, packed_modules_list: List,
                           model_config=None) -> bool:
         w = getattr(source_layer, "weight", None)
+        if isinstance(source_layer, (nn.Embedding, BaseLayerWithDelta)):
+            return False
         return isinstance(w, torch.Tensor) and w.dim() == 2 and len(packed_modules_list) == cls._n_packed
 
 

@@ -127,6 +127,41 @@ def segment(indices: torch.Tensor, num_slots: int):
     return perm, off
 
 
+def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_ids: torch.Tensor,
+            max_deltas: int, vocab_size: int, extra_vocab_size: int, base_indices: torch.Tensor,
+            sampler_indices: Optional[torch.Tensor] = None,
+            sampler_indices_padded: Optional[torch.Tensor] = None,
+            embeddings_indices: Optional[torch.Tensor] = None,
+            n_missing: Optional[torch.Tensor] = None) -> None:
+    """Delta ids -> slot indices on the device, written into the given int64 tensors (the index
+    tensors of convert_mapping, serving/vllm/delta/models.py:69-145).  token_ids [T], prompt_ids [P]
+    or None, slot_ids [S]: int64 on the GPU; the outputs are the manager's persistent buffers
+    (at least T resp. P long; embeddings_indices [2, >= T])."""
+    _need_cuda(token_ids, prompt_ids, slot_ids, base_indices, sampler_indices, sampler_indices_padded,
+               embeddings_indices, n_missing)
+    for t in (token_ids, prompt_ids, slot_ids, base_indices, sampler_indices, sampler_indices_padded,
+              embeddings_indices):
+        if t is not None and t.dtype != torch.int64:
+            raise ValueError("id and index tensors must be int64")
+    T = token_ids.numel()
+    P = 0 if prompt_ids is None else prompt_ids.numel()
+    if base_indices.numel() < T or (P and (sampler_indices is None or sampler_indices.numel() < P)):
+        raise ValueError("index buffers are shorter than the batch")
+    if sampler_indices_padded is not None and sampler_indices_padded.numel() < P:
+        raise ValueError("index buffers are shorter than the batch")
+    ld = 0
+    if embeddings_indices is not None:
+        if embeddings_indices.dim() != 2 or embeddings_indices.shape[0] != 2 or embeddings_indices.stride(1) != 1:
+            raise ValueError("embeddings_indices must be [2, n] with contiguous rows")
+        ld = embeddings_indices.stride(0)
+    ptr = lambda t: None if t is None else t.data_ptr()
+    rc = _lib.lib().dz_map_ids(token_ids.data_ptr(), T, ptr(prompt_ids), P, slot_ids.data_ptr(),
+                               slot_ids.numel(), max_deltas, vocab_size, extra_vocab_size,
+                               base_indices.data_ptr(), ptr(sampler_indices), ptr(sampler_indices_padded),
+                               ptr(embeddings_indices), ld, ptr(n_missing), _stream())
+    _lib.check(rc, "dz_map_ids")
+
+
 # ---------------------------------------------------------------------------------------------
 # workspace: zero-filled once per device, reused by every call on that device
 # ---------------------------------------------------------------------------------------------

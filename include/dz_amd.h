@@ -42,6 +42,7 @@ extern "C" {
 
 #define DZ_MAX_TOKENS_FUSED 128   /* largest T the fused decode kernel takes in one launch   */
 #define DZ_MAX_SLOTS_SEGMENT 768   /* largest S dz_segment takes (its tables live in LDS)      */
+#define DZ_MAX_SLOTS_MAP 4096      /* largest S dz_map_ids takes (the slot table lives in LDS) */
 
 /* Library version (major*10000 + minor*100 + patch). */
 int dz_version(void);
@@ -79,6 +80,24 @@ int dz_merge(const uint16_t* w_base, const void* codes, const void* meta, const 
  * Ids outside [-1, S) are treated as -1; S <= DZ_MAX_SLOTS_SEGMENT.  (The reference's scheduler sorts the batch by delta
  * id, serving/vllm/core/scheduler.py:101-104; this makes the op independent of that.) */
 int dz_segment(const int64_t* indices, int T, int S, int32_t* perm, int32_t* seg_off, void* stream);
+
+/* Delta id -> slot index for a batch, on the device: the index tensors the reference's manager
+ * builds in a Python loop over tokens (convert_mapping, serving/vllm/delta/models.py:69-145).
+ * token_ids [T] and prompt_ids [P] hold delta ids (<= 0: base model); slot_ids [S] holds the id
+ * resident in each slot (<= 0: free).  Writes
+ *   base_indices[t]            = slot of token_ids[t], -1 for the base model
+ *   sampler_indices[p]         = slot of prompt_ids[p], -1 for the base model
+ *   sampler_indices_padded[p]  = p + (slot == -1 ? max_deltas - 1 : slot) * P
+ *   embeddings_indices[0][t]   = e * extra_vocab_size, [1][t] = e * (vocab_size + extra_vocab_size),
+ *                                e = slot for a delta and 0 for the base model, a result of -1
+ *                                replaced by max_deltas - 1 (row stride ld_emb elements)
+ * as the reference does.  sampler_indices_padded, embeddings_indices and n_missing may be NULL; P
+ * may be 0.  An id > 0 that is in no slot maps to -1 and, when n_missing is given, adds one to
+ * *n_missing (the caller zeroes it), where the reference's list.index raises.  S <= DZ_MAX_SLOTS_MAP. */
+int dz_map_ids(const int64_t* token_ids, int T, const int64_t* prompt_ids, int P,
+               const int64_t* slot_ids, int S, int max_deltas, int vocab_size, int extra_vocab_size,
+               int64_t* base_indices, int64_t* sampler_indices, int64_t* sampler_indices_padded,
+               int64_t* embeddings_indices, int ld_emb, int32_t* n_missing, void* stream);
 
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
  * zero-filled once before first use; calls leave it ready for the next call.  Calls that share

@@ -15,6 +15,7 @@ Pinning status (what independent evidence each function is checked against in te
   forward_ref                   per-token python loop, F.linear special cases          (pinned)
   native layout functions       defined by this project; pinned by round trip through
                                 dequant_gptq
+  convert_mapping_ref           hand-computed index tensors for small batches          (pinned)
 The fused third-party kernel the reference calls on the serving path (triteia
 `sbmm_4bit_2_4_native`, un-vendored and un-pinned: scripts/install.sh:2, call site
 serving/vllm/delta/deltazip_marlin.py:18) cannot be inspected: its bit layout and rounding are
@@ -391,6 +392,35 @@ def dequant_native(codes, meta, scales16, k, n, bits) -> np.ndarray:
                         # positions are distinct within a group, so plain assignment is safe.
                         out[rows, cols] = val
     return out
+
+
+# --------------------------------------------------------------------------------------
+# a11: delta id -> slot index tensors (serving/vllm/delta/models.py:69-145)
+# --------------------------------------------------------------------------------------
+
+
+def convert_mapping_ref(index_mapping, prompt_mapping, delta_index_to_id, max_deltas, vocab_size,
+                        extra_vocab_size):
+    """Returns (base_indices [T], sampler_indices [P], sampler_indices_padded [P],
+    embeddings_indices [2, T]) as int64 arrays.  `max_deltas` is what the caller passes there
+    (the manager passes slots + 1, models.py:401).
+
+    models.py:106-116: slot = delta_index_to_id.index(id) for id > 0 (raises ValueError when the
+    id is in no slot), else -1; the embedding index uses 0 instead of -1 for the base model.
+    models.py:122-126: embeddings_indices = [e * extra_vocab, e * (vocab + extra_vocab)], entries
+    equal to -1 replaced by max_deltas - 1.  models.py:129-133: padded = arange(P) + s' * P with
+    s' = s, or max_deltas - 1 where s == -1."""
+    table = list(delta_index_to_id)
+    slot = lambda x: table.index(x) if x > 0 else -1
+    base = np.array([slot(x) for x in index_mapping], dtype=np.int64)
+    emb = np.array([slot(x) if x > 0 else 0 for x in index_mapping], dtype=np.int64)
+    sampler = np.array([slot(x) for x in prompt_mapping], dtype=np.int64)
+    emb2 = np.stack([emb * extra_vocab_size, emb * (vocab_size + extra_vocab_size)]).astype(np.int64)
+    emb2[emb2 == -1] = max_deltas - 1
+    padded = sampler.copy()
+    padded[padded == -1] = max_deltas - 1
+    padded = np.arange(len(padded), dtype=np.int64) + padded * len(padded)
+    return base, sampler, padded, emb2
 
 
 # --------------------------------------------------------------------------------------

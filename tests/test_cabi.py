@@ -55,6 +55,12 @@ def test_argument_checks_happen_on_the_host(dzlib):
     assert dzlib.dz_merge(None, one, one, one, 512, 64, 4, -1, one, None) == -1
     assert dzlib.dz_segment(None, 4, 2, one, one, None) == -1
     assert dzlib.dz_segment(one, 0, 2, one, one, None) == -2
+    mp = dzlib.dz_map_ids
+    assert mp(None, 4, None, 0, one, 2, 3, 100, 0, one, None, None, None, 0, None, None) == -1
+    assert mp(one, 4, None, 2, one, 2, 3, 100, 0, one, None, None, None, 0, None, None) == -1
+    assert mp(one, 0, None, 0, one, 2, 3, 100, 0, one, None, None, None, 0, None, None) == -2
+    assert mp(one, 4, None, 0, one, 5000, 3, 100, 0, one, None, None, None, 0, None, None) == -2
+    assert mp(one, 4, None, 0, one, 2, 3, 100, 0, one, None, None, one, 3, None, None) == -2
     assert dzlib.dz_gemm_f16(one, one, one, 8, 100, 128, 0, 128, None) == -2
     assert dzlib.dz_gemm_f16(None, one, one, 8, 128, 128, 0, 128, None) == -1
 

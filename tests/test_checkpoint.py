@@ -1,0 +1,143 @@
+"""Checkpoint reader and converter: a synthetic delta checkpoint in the reference's on-disk format
+(deltazip/modeling/_base.py:596-645: GPTQ-style keys in deltazip-compressed.safetensors +
+compress_config.json) is read, fused and converted to the native layout; every module must
+dequantise, bit for bit, to what the reference's dequantisation gives for the separate modules."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import dz_oracle as o
+from deltazip_amd import checkpoint as ck
+
+H, I, V = 256, 512, 64        # hidden, intermediate, vocabulary of the toy model
+SHAPES = {"self_attn.q_proj": (H, H), "self_attn.k_proj": (64, H), "self_attn.v_proj": (64, H),
+          "self_attn.o_proj": (H, H), "mlp.gate_proj": (I, H), "mlp.up_proj": (I, H), "mlp.down_proj": (H, I)}
+
+
+def make_state_dict(bits, gs, layers=2, seed=100):
+    sd, ref = {}, {}
+    for layer in range(layers):
+        for j, (name, (n, k)) in enumerate(SHAPES.items()):
+            d = o.make_delta(n, k, 1e-3, bits, gs, seed + 10 * layer + j)
+            mod = f"model.layers.{layer}.{name}"
+            for key in ("qweight", "qzeros", "scales", "g_idx"):
+                sd[f"{mod}.{key}"] = torch.from_numpy(d[key].copy())
+            ref[mod] = o.dequant_gptq(d["qweight"], d["qzeros"], d["scales"], d["g_idx"], bits).T  # [N, K]
+        for name in ("input_layernorm", "post_attention_layernorm"):
+            sd[f"model.layers.{layer}.{name}.weight"] = torch.full((H,), 0.5 + layer, dtype=torch.float16)
+    sd["model.embed_tokens.weight"] = torch.arange(V * H, dtype=torch.float32).reshape(V, H).half()
+    sd["lm_head.weight"] = torch.ones(V, H, dtype=torch.float16)
+    sd["model.norm.weight"] = torch.ones(H, dtype=torch.float16)
+    return sd, ref
+
+
+def native_dequant(q, m, s, k, bits):
+    n = s.shape[1]
+    qn = q.numpy().view(np.uint32)
+    codes = qn.reshape(n // 32, k // 256, 64, 4) if bits == 2 else qn.reshape(n // 32, k // 256, 2, 64, 4)
+    meta = m.numpy().view(np.uint32).reshape(n // 32, k // 256, 64, 4)
+    return o.dequant_native(codes, meta, s.numpy(), k, n, bits)
+
+
+@pytest.mark.parametrize("bits,gs", [(4, -1), (2, -1), (4, 128)])
+def test_convert_model_fuses_and_keeps_values(dzlib, bits, gs):
+    sd, ref = make_state_dict(bits, gs)
+    out = ck.convert_model(sd, bits=bits)
+    for layer in range(2):
+        p = f"model.layers.{layer}."
+        fused = {"self_attn.qkv_proj": ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"],
+                 "mlp.gate_up_proj": ["mlp.gate_proj", "mlp.up_proj"],
+                 "self_attn.o_proj": ["self_attn.o_proj"], "mlp.down_proj": ["mlp.down_proj"]}
+        for target, parts in fused.items():
+            want = np.concatenate([ref[p + x] for x in parts], axis=0)
+            n, k = want.shape
+            q, m, s = (out[f"{p}{target}.0.{x}"] for x in ("qweight", "meta", "scales"))
+            pf = 32 // bits
+            assert tuple(q.shape) == (k // (pf * 4), 2 * n) and tuple(m.shape) == (n, k // 16)
+            assert tuple(s.shape) == (1 if gs == -1 else k // gs, n)
+            got = native_dequant(q, m, s, k, bits)
+            assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(want).view(np.uint16)), target
+        # the separate projections are gone, the layer norms are carried over
+        assert f"{p}self_attn.q_proj.0.qweight" not in out
+        assert torch.equal(out[f"{p}input_layernorm.0.weight"], sd[f"{p}input_layernorm.weight"])
+    assert torch.equal(out["model.embed_tokens.0.weight"], sd["model.embed_tokens.weight"])
+    assert torch.equal(out["lm_head.0.weight"], sd["lm_head.weight"])
+    assert not any(k.endswith((".qzeros", ".g_idx")) for k in out)
+
+
+def test_bits_are_read_off_the_shapes(dzlib):
+    for bits in (2, 4):
+        sd, _ = make_state_dict(bits, -1, layers=1)
+        a = ck.convert_model(sd)             # no bits given
+        b = ck.convert_model(sd, bits=bits)
+        assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)
+
+
+def test_missing_part_of_a_fused_module_is_an_error(dzlib):
+    sd, _ = make_state_dict(4, -1, layers=1)
+    for key in ("qweight", "qzeros", "scales", "g_idx"):
+        del sd[f"model.layers.0.self_attn.k_proj.{key}"]
+    with pytest.raises(ValueError, match="missing parts"):
+        ck.convert_model(sd, bits=4)
+
+
+def test_compression_config_round_trip(tmp_path):
+    cfg = ck.CompressionConfig(bits=2, sparsity=0.5, prunen=2, prunem=4, group_size=-1)
+    cfg.save_pretrained(str(tmp_path))
+    with open(tmp_path / "compress_config.json") as f:
+        raw = json.load(f)
+    assert raw["bits"] == 2 and raw["prunen"] == 2 and raw["prunem"] == 4 and raw["lossless"] == "none"
+    back = ck.CompressionConfig.from_pretrained(str(tmp_path))
+    assert back.to_dict() == cfg.to_dict() and back.pack_factor == 16
+    with pytest.raises(ValueError):
+        ck.CompressionConfig(bits=5)
+    with pytest.raises(ValueError):
+        ck.CompressionConfig(sparsity=1.5)
+    with pytest.raises(ValueError):
+        ck.CompressionConfig(group_size=0)
+
+
+@pytest.mark.parametrize("converted_on_disk", [False, True])
+def test_delta_model_from_checkpoint(dzlib, tmp_path, converted_on_disk):
+    from safetensors.torch import save_file
+    bits = 4
+    sd, ref = make_state_dict(bits, -1)
+    cfg = ck.CompressionConfig(bits=bits, sparsity=0.5, prunen=2, prunem=4)
+    if converted_on_disk:
+        ck.save_converted(ck.convert_model(sd, bits=bits), cfg, str(tmp_path))
+    else:
+        save_file(sd, os.path.join(tmp_path, ck.CHECKPOINT_NAME))
+        cfg.save_pretrained(str(tmp_path))
+    dm = ck.DeltaModel.from_checkpoint(str(tmp_path), id=7, pin_memory=False)
+    assert dm.id == 7 and dm.bitwidth == bits
+    names = set(dm.deltas)
+    assert "model.layers.1.self_attn.qkv_proj" in names and "model.layers.0.mlp.gate_up_proj" in names
+    assert "lm_head" in names and "model.embed_tokens" in names and "model.norm" in names
+    assert not any(x.endswith(("q_proj", "k_proj", "v_proj", "gate_proj", "up_proj")) and "qkv" not in x
+                   and "gate_up" not in x for x in names)
+    d = dm.get_delta("model.layers.1.mlp.down_proj")
+    assert d._compressed and d.meta is not None and d.qzeros is None
+    got = native_dequant(d.qweight, d.meta, d.scales, I, bits)
+    assert np.array_equal(got, ref["model.layers.1.mlp.down_proj"])
+    e = dm.get_delta("model.embed_tokens")
+    assert not e._compressed and torch.equal(e.weight, sd["model.embed_tokens.weight"])
+    assert dm.get_delta("nope") is None
+
+
+def test_unsupported_checkpoints_are_refused(dzlib):
+    sd, _ = make_state_dict(4, -1, layers=1)
+    with pytest.raises(NotImplementedError):
+        ck.DeltaModel.from_tensors(sd, 1, ck.CompressionConfig(bits=4, lossless="gdeflate"))
+    with pytest.raises(NotImplementedError):
+        ck.DeltaModel.from_tensors(sd, 1, ck.CompressionConfig(bits=8))
+    # a dense (not 2:4) delta: the repacker's check fires
+    k, n = 256, 32
+    codes = np.full((k, n), 9, dtype=np.uint8)
+    qw, qz, sc, gi = o.pack_codes_gptq(codes, np.full((1, n), 8), np.full((1, n), 0.5, np.float16), 4)
+    bad = {"model.layers.0.self_attn.o_proj." + key: torch.from_numpy(v.copy())
+           for key, v in (("qweight", qw), ("qzeros", qz), ("scales", sc), ("g_idx", gi))}
+    with pytest.raises(ValueError):
+        ck.convert_model(bad, bits=4)

@@ -1,0 +1,261 @@
+"""Slot manager: bookkeeping on the CPU (no kernels), the oracle's convert_mapping restatement
+against hand-computed answers, and on the GPU the device-side mapping and a checkpoint -> manager
+-> layer forward pass checked against the oracle."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+from oracle import dz_oracle as o
+from deltazip_amd import (DeltaConfig, DeltaMapping, DeltaModel, CompressionConfig, LRUCacheDeltaModelManager,
+                          DeltaModelManager, create_delta_manager, convert_model)
+from deltazip_amd.layers import (MergedQKVParallelLinearWithDelta, MergedColumnParallelLinearWithDelta,
+                                 RowParallelLinearWithDelta)
+from deltazip_amd.manager import LRUCache
+
+H, I, V = 256, 512, 64
+
+
+class Attn(nn.Module):
+    def __init__(self, dev):
+        super().__init__()
+        self.qkv_proj = nn.Linear(H, H + 128, bias=False, dtype=torch.float16, device=dev)
+        self.o_proj = nn.Linear(H, H, bias=False, dtype=torch.float16, device=dev)
+
+
+class Mlp(nn.Module):
+    def __init__(self, dev):
+        super().__init__()
+        self.gate_up_proj = nn.Linear(H, 2 * I, bias=False, dtype=torch.float16, device=dev)
+        self.down_proj = nn.Linear(I, H, bias=False, dtype=torch.float16, device=dev)
+
+
+class Block(nn.Module):
+    def __init__(self, dev):
+        super().__init__()
+        self.self_attn, self.mlp = Attn(dev), Mlp(dev)
+
+
+class Inner(nn.Module):
+    def __init__(self, dev, layers):
+        super().__init__()
+        self.embed_tokens = nn.Embedding(V, H, dtype=torch.float16, device=dev)
+        self.layers = nn.ModuleList([Block(dev) for _ in range(layers)])
+
+
+class ToyModel(nn.Module):
+    """Module tree and class attributes shaped like the serving model
+    (model_executor/models/llama.py:299-340)."""
+    packed_modules_mapping = {"qkv_proj": ["q_proj", "k_proj", "v_proj"], "gate_up_proj": ["gate_proj", "up_proj"]}
+    supported_delta_modules = ["qkv_proj", "o_proj", "gate_up_proj", "down_proj", "embed_tokens", "lm_head"]
+
+    def __init__(self, dev="cpu", layers=1):
+        super().__init__()
+        self.model = Inner(dev, layers)
+        self.lm_head = nn.Linear(H, V, bias=False, dtype=torch.float16, device=dev)
+        with torch.no_grad():
+            g = torch.Generator().manual_seed(5)
+            for p in self.parameters():
+                p.copy_((torch.randn(p.shape, generator=g) * 0.02).to(p.dtype))
+
+
+SHAPES = {"self_attn.q_proj": (H, H), "self_attn.k_proj": (64, H), "self_attn.v_proj": (64, H),
+          "self_attn.o_proj": (H, H), "mlp.gate_proj": (I, H), "mlp.up_proj": (I, H), "mlp.down_proj": (H, I)}
+
+
+def make_delta_model(delta_id, bits, seed):
+    """A DeltaModel built the way a checkpoint is read, plus the reference dequantisation [N, K] of
+    every fused module."""
+    sd, ref = {}, {}
+    for j, (name, (n, k)) in enumerate(SHAPES.items()):
+        d = o.make_delta(n, k, 1e-3, bits, -1, seed + j)
+        for key in ("qweight", "qzeros", "scales", "g_idx"):
+            sd[f"model.layers.0.{name}.{key}"] = torch.from_numpy(d[key].copy())
+        ref[name] = o.dequant_gptq(d["qweight"], d["qzeros"], d["scales"], d["g_idx"], bits)   # [K, N]
+    fused = {"self_attn.qkv_proj": np.concatenate([ref[f"self_attn.{x}_proj"] for x in "qkv"], axis=1),
+             "self_attn.o_proj": ref["self_attn.o_proj"],
+             "mlp.gate_up_proj": np.concatenate([ref["mlp.gate_proj"], ref["mlp.up_proj"]], axis=1),
+             "mlp.down_proj": ref["mlp.down_proj"]}
+    dm = DeltaModel.from_tensors(sd, delta_id, CompressionConfig(bits=bits, prunen=2, prunem=4, sparsity=0.5),
+                                 pin_memory=False)
+    return dm, fused
+
+
+# ---------------------------------------------------------------------------------------------
+# CPU
+# ---------------------------------------------------------------------------------------------
+def test_oracle_convert_mapping_known_answers():
+    # slots: [id 7, free, id 3]; manager passes max_deltas = slots + 1 = 4
+    base, samp, padded, emb = o.convert_mapping_ref((3, 3, 0, 7, 0), (3, 0, 7), [7, None, 3], 4, 100, 10)
+    assert base.tolist() == [2, 2, -1, 0, -1]
+    assert samp.tolist() == [2, -1, 0]
+    assert padded.tolist() == [0 + 2 * 3, 1 + 3 * 3, 2 + 0 * 3]
+    assert emb.tolist() == [[20, 20, 0, 0, 0], [220, 220, 0, 0, 0]]
+    with pytest.raises(ValueError):
+        o.convert_mapping_ref((5,), (), [7, None, 3], 4, 100, 0)
+
+
+def test_lru_cache_order_and_callbacks():
+    removed = []
+
+    class C(LRUCache):
+        def _on_remove(self, key, value):
+            removed.append(key)
+
+    c = C(2)
+    c.put(1, "a"); c.put(2, "b"); c.get(1); c.put(3, "c")          # 2 is the oldest now
+    assert removed == [2] and list(c.keys()) == [1, 3] and len(c) == 2
+    c.touch(1); c.remove_oldest()
+    assert removed == [2, 3] and 1 in c
+    assert c.pop(1) == "a" and removed == [2, 3, 1] and c.pop(9, "x") == "x"
+
+
+def test_manager_wraps_modules_and_tracks_slots(dzlib):
+    model = ToyModel()
+    cfg = DeltaConfig(max_deltas=2, max_bitwidth=4, max_cpu_deltas=3)
+    mgr = create_delta_manager(model, 8, 64, V, cfg)
+    assert isinstance(model.model.layers[0].self_attn.qkv_proj, MergedQKVParallelLinearWithDelta)
+    assert isinstance(model.model.layers[0].mlp.gate_up_proj, MergedColumnParallelLinearWithDelta)
+    assert isinstance(model.model.layers[0].mlp.down_proj, RowParallelLinearWithDelta)
+    assert isinstance(model.model.embed_tokens, nn.Embedding)         # not wrapped: outside this path
+    assert sorted(mgr.modules) == ["model.layers.0.mlp.down_proj", "model.layers.0.mlp.gate_up_proj",
+                                   "model.layers.0.self_attn.o_proj", "model.layers.0.self_attn.qkv_proj"]
+    assert mgr.packed_modules["model.layers.0.self_attn.qkv_proj"] == [
+        "model.layers.0.self_attn.q_proj", "model.layers.0.self_attn.k_proj", "model.layers.0.self_attn.v_proj"]
+    qkv = model.model.layers[0].self_attn.qkv_proj
+    assert qkv.indices is mgr.base_indices and qkv.indices_len is mgr.indices_len
+    assert model.delta_manager is mgr and mgr.capacity == 3 and mgr.delta_slots == 2
+
+    dms = [make_delta_model(i, 4, 10 * i)[0] for i in (1, 2, 3)]
+    assert [mgr.add_delta(d) for d in dms] == [True, True, True] and not mgr.add_delta(dms[0])
+    with pytest.raises(RuntimeError, match="No free Delta slots"):
+        mgr.add_delta(make_delta_model(4, 4, 40)[0])
+    assert len(mgr) == 3 and set(mgr.list_deltas()) == {1, 2, 3} and mgr.get_delta(2) is dms[1]
+    assert mgr.activate_delta(2) and not mgr.activate_delta(2) and mgr.activate_delta(1)
+    assert mgr.delta_index_to_id == [2, 1]
+    with pytest.raises(ValueError, match="No free delta slots"):
+        mgr.activate_delta(3)
+    # slot 0 of the fused qkv layer holds delta 2's tensors
+    want = dms[1].get_delta("model.layers.0.self_attn.qkv_proj")
+    assert torch.equal(qkv.qweight_stacked[0].reshape(-1), want.qweight.reshape(-1))
+    assert torch.equal(qkv.scales_stacked[0].reshape(-1), want.scales.reshape(-1))
+    assert mgr.deactivate_delta(2) and not mgr.deactivate_delta(2)
+    assert mgr.delta_index_to_id == [None, 1]
+    assert mgr.activate_delta(3) and mgr.delta_index_to_id == [3, 1]
+    assert mgr.remove_delta(1) and mgr.delta_index_to_id == [3, None] and not mgr.remove_delta(1)
+    mgr.remove_all_deltas()
+    assert len(mgr) == 0 and mgr.delta_index_to_id == [None, None]
+    # there is no CPU implementation of the mapping kernel
+    with pytest.raises(ValueError, match="GPU"):
+        mgr.set_delta_mapping(DeltaMapping((0, 0), (0,)))
+
+
+def test_lru_manager_evicts_least_recently_used(dzlib):
+    model = ToyModel()
+    mgr = create_delta_manager(model, 8, 64, V, DeltaConfig(max_deltas=2, max_bitwidth=4, max_cpu_deltas=3),
+                               delta_manager_cls=LRUCacheDeltaModelManager)
+    for i in (1, 2, 3):
+        assert mgr.add_delta(make_delta_model(i, 4, 10 * i)[0])
+    assert not mgr.add_delta(mgr.get_delta(1))
+    mgr.activate_delta(1); mgr.activate_delta(2)
+    assert mgr.delta_index_to_id == [1, 2]
+    mgr.activate_delta(1)                       # touch: 2 is now the least recently used
+    mgr.activate_delta(3)
+    assert mgr.delta_index_to_id == [1, 3]
+    # host cache is full: the registered delta that was looked up longest ago (1: the second
+    # activate_delta(1) returned before reading it) goes, and leaves its GPU slot as well
+    mgr.add_delta(make_delta_model(4, 4, 40)[0])
+    assert len(mgr) == 3 and set(mgr.list_deltas()) == {2, 3, 4} and mgr.delta_index_to_id == [None, 3]
+    assert mgr.remove_oldest_delta() and len(mgr) == 2
+
+
+def test_model_without_delta_support_is_refused():
+    with pytest.raises(ValueError, match="not supported"):
+        create_delta_manager(nn.Linear(4, 4), 1, 8, 10, DeltaConfig())
+
+
+# ---------------------------------------------------------------------------------------------
+# GPU
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,P,S", [(1, 1, 1), (5, 3, 3), (37, 37, 8), (300, 7, 64), (4096, 129, 700)])
+def test_map_ids_matches_reference_loop(dev, T, P, S):
+    from deltazip_amd import ops
+    rng = np.random.default_rng(T + S)
+    table = [None] * S
+    resident = rng.choice(np.arange(1, 10 * S + 2), size=max(1, (2 * S) // 3), replace=False).tolist()
+    for s_, d in zip(rng.permutation(S)[: len(resident)], resident):
+        table[int(s_)] = int(d)
+    pool = np.array(resident + [0, 0, -1])
+    tok = rng.choice(pool, size=T).astype(np.int64)
+    prm = rng.choice(pool, size=P).astype(np.int64)
+    vocab, extra = 32000, 3
+    tok_nonneg, prm_nonneg = np.maximum(tok, 0), np.maximum(prm, 0)
+    want = o.convert_mapping_ref(tok_nonneg.tolist(), prm_nonneg.tolist(), table, S + 1, vocab, extra)
+    n = T + 11
+    base = torch.full((n,), -7, dtype=torch.long, device=dev)
+    samp, padded = torch.full_like(base, -7), torch.full_like(base, -7)
+    emb = torch.full((2, n), -7, dtype=torch.long, device=dev)
+    missing = torch.zeros(1, dtype=torch.int32, device=dev)
+    slots = torch.tensor([d if d is not None else 0 for d in table], dtype=torch.long, device=dev)
+    ops.map_ids(torch.from_numpy(tok).to(dev), torch.from_numpy(prm).to(dev), slots, S + 1, vocab, extra,
+                base, samp, padded, emb, missing)
+    torch.cuda.synchronize()
+    assert np.array_equal(base[:T].cpu().numpy(), want[0]) and np.array_equal(samp[:P].cpu().numpy(), want[1])
+    assert np.array_equal(padded[:P].cpu().numpy(), want[2]) and np.array_equal(emb[:, :T].cpu().numpy(), want[3])
+    # nothing written past the batch, nothing reported missing
+    assert (base[T:] == -7).all() and (samp[P:] == -7).all() and (emb[:, T:] == -7).all()
+    assert int(missing.item()) == 0
+    # an id that is in no slot: -1 and counted
+    tok2 = torch.tensor([10 * S + 5], dtype=torch.long, device=dev)
+    ops.map_ids(tok2, None, slots, S + 1, vocab, extra, base, n_missing=missing)
+    torch.cuda.synchronize()
+    assert int(base[0].item()) == -1 and int(missing.item()) == 1
+
+
+@pytest.mark.gpu
+def test_checkpoint_to_manager_to_forward(dev):
+    bits = 4
+    model = ToyModel(dev)
+    base = {n: m.weight.detach().cpu().numpy().copy() for n, m in model.named_modules()
+            if isinstance(m, nn.Linear)}
+    mgr = create_delta_manager(model, 8, 64, V, DeltaConfig(max_deltas=3, max_bitwidth=bits, max_cpu_deltas=4),
+                               delta_manager_cls=LRUCacheDeltaModelManager)
+    fused = {}
+    for did in (11, 12, 13, 14):
+        dm, fused[did] = make_delta_model(did, bits, 100 * did)
+        mgr.add_delta(dm)
+    for did in (12, 11, 13):
+        mgr.activate_delta(did)
+    assert mgr.delta_index_to_id == [12, 11, 13]
+    ids = (11, 11, 0, 13, 12, 12, 0, 13, 11)
+    x = torch.from_numpy(o.make_x(len(ids), H, 3)).to(dev)
+
+    def check(ids):
+        mgr.set_delta_mapping(DeltaMapping(ids, ids[:2]))
+        torch.cuda.synchronize()
+        slots = [mgr.delta_index_to_id.index(i) if i > 0 else -1 for i in ids]
+        assert mgr.base_indices[: len(ids)].tolist() == slots and list(mgr.indices_len) == [len(ids), 2, 2, len(ids)]
+        for name in ("self_attn.qkv_proj", "self_attn.o_proj", "mlp.gate_up_proj"):
+            layer = model.get_submodule("model.layers.0." + name)
+            y, bias = layer(x)
+            torch.cuda.synchronize()
+            table = {i: fused[i][name] for i in fused}
+            uniq = sorted({i for i in ids if i > 0})
+            ref = o.forward_ref(x.cpu().numpy(), base["model.layers.0." + name], [table[i] for i in uniq],
+                                np.array([uniq.index(i) if i > 0 else -1 for i in ids]))
+            assert bias is None and o.rel_err(y.float().cpu().numpy(), ref) <= 1e-2, name
+
+    check(ids)
+    # delta 14 takes the least recently used slot (12's: 11 and 13 were activated after it)
+    mgr.activate_delta(14)
+    assert mgr.delta_index_to_id == [14, 11, 13]
+    check((14, 11, 0, 13, 14, 14, 0, 13, 11))
+    with pytest.raises(ValueError, match="not in list"):
+        mgr.set_delta_mapping(DeltaMapping((12, 0), (12,)))
+    # an unchanged mapping is not converted again
+    m = DeltaMapping((11, 0), (11,))
+    mgr.set_delta_mapping(m)
+    before = mgr._staged
+    mgr.set_delta_mapping(DeltaMapping((11, 0), (11,)))
+    assert mgr._last_mapping == m and mgr._staged is before
