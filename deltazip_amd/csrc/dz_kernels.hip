@@ -199,6 +199,31 @@ __global__ __launch_bounds__(256) void dz_map_ids_kernel(const long long* __rest
 }
 
 // ---------------------------------------------------------------------------------------------
+// embedding rows picked from the base table or from a delta's own table, per token.
+// One workgroup per token; 16 bytes per lane and step.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void dz_embedding_select_kernel(const long long* __restrict__ tokens,
+                                                                  const long long* __restrict__ idx,
+                                                                  const _Float16* __restrict__ base,
+                                                                  const _Float16* __restrict__ stack,
+                                                                  long long stack_stride, int S, int V,
+                                                                  int H, _Float16* __restrict__ out,
+                                                                  int ldo) {
+  const int t = blockIdx.x;
+  const long long tok = tokens[t];
+  const long long id = idx[t];
+  const _Float16* table = (id >= 0 && id < S) ? stack + id * stack_stride : base;
+  u4_t* dst = (u4_t*)(out + (size_t)t * ldo);
+  const bool valid = tok >= 0 && tok < V && table != nullptr;
+  const u4_t* src = (const u4_t*)(table + (valid ? (size_t)tok * H : 0));
+  for (int c = threadIdx.x; c < H / 8; c += 256) {
+    u4_t v = {0u, 0u, 0u, 0u};
+    if (valid) v = src[c];
+    dst[c] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 int g_ksplit_override = 0;
@@ -305,6 +330,20 @@ int dz_map_ids(const int64_t* token_ids, int T, const int64_t* prompt_ids, int P
                      P, (const long long*)slot_ids, S, (long long)max_deltas - 1, (long long)vocab_size,
                      (long long)extra_vocab_size, (long long*)base_indices, (long long*)sampler_indices,
                      (long long*)sampler_indices_padded, (long long*)embeddings_indices, ld_emb, n_missing);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+int dz_embedding_select(const int64_t* tokens, const int64_t* indices, const uint16_t* base_weight,
+                        const uint16_t* weight_stack, long long stack_stride, int S, uint16_t* out, int T,
+                        int V, int H, int ldo, void* stream) {
+  if (!tokens || !indices || !out || (!base_weight && !weight_stack)) return DZ_EINVAL;
+  if (T < 1 || V < 1 || H < 8 || H % 8 || ldo < H || ldo % 8 || S < 0 || (S > 0 && !weight_stack)) return DZ_ESHAPE;
+  if (((uintptr_t)base_weight & 15) || ((uintptr_t)weight_stack & 15) || ((uintptr_t)out & 15) ||
+      (stack_stride & 7))
+    return DZ_EALIGN;
+  hipLaunchKernelGGL(dz_embedding_select_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream,
+                     (const long long*)tokens, (const long long*)indices, (const _Float16*)base_weight,
+                     (const _Float16*)weight_stack, stack_stride, S, V, H, (_Float16*)out, ldo);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 

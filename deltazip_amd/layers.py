@@ -177,8 +177,127 @@ class RowParallelLinearWithDelta(LinearWithDelta):
         return super().apply_weights(x, None)
 
 
-_all_delta_classes = (ColumnParallelLinearWithDelta, MergedColumnParallelLinearWithDelta,
+class VocabParallelEmbeddingWithDelta(BaseLayerWithDelta):
+    """Embedding whose table is replaced, per token, by the token's delta's own table
+    (layers_marlin.py:97-171).  The base layer is any module with a fp16 `weight` [vocab, hidden]
+    (torch.nn.Embedding fits)."""
+
+    def __init__(self, base_layer: nn.Module) -> None:
+        super().__init__()
+        self.base_layer = base_layer
+        self.indices: Optional[torch.Tensor] = None
+        self.indices_len: Optional[List[int]] = None
+
+    def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
+        w = self.base_layer.weight
+        if w.dtype != torch.float16 or w.dim() != 2:
+            raise ValueError("base embedding weight must be float16 [vocab, hidden]")
+        vocab = getattr(self.base_layer, "org_vocab_size", w.shape[0])
+        self.delta_weights = torch.zeros((max_deltas, vocab, w.shape[1]), dtype=w.dtype, device=w.device)
+        self.bitwidth = [0] * max_deltas
+
+    def reset_delta(self, index: int):
+        self.bitwidth[index] = 0
+        self.delta_weights[index] = 0
+
+    def set_delta(self, index: int, bitwidth: int, weight: torch.Tensor, *unused):
+        self.bitwidth[index] = bitwidth
+        self.delta_weights[index].copy_(weight, non_blocking=ASYNC_COPY)
+
+    def set_mapping(self, base_indices: torch.Tensor, sampler_indices=None, sampler_indices_padded=None,
+                    embeddings_indices=None, indices_len: Optional[List[int]] = None):
+        self.indices = base_indices
+        self.embeddings_indices = embeddings_indices
+        self.indices_len = indices_len if indices_len is not None else [base_indices.numel()]
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.apply_delta_embed(x, self.delta_weights, self.indices[: self.indices_len[0]],
+                                     self.base_layer.weight)
+
+    @classmethod
+    def can_replace_layer(cls, source_layer: nn.Module, delta_config: DeltaConfig, packed_modules_list: List,
+                          model_config=None) -> bool:
+        return type(source_layer) is nn.Embedding
+
+
+class LogitsProcessorWithDelta(BaseLayerWithDelta):
+    """Output projection with one full [vocab, hidden] weight per delta (layers_marlin.py:614-725):
+    a sampled row multiplies its delta's weight, or the base `embedding` passed to `_get_logits`
+    when it has none.  `base_layer` only has to provide `vocab_size`; when it has a `forward` of
+    its own (the serving engine's LogitsProcessor), `forward` defers to it with this object in
+    place of `self`, as the reference does."""
+
+    def __init__(self, base_layer, hidden_size: int, dtype: torch.dtype, device: torch.device) -> None:
+        super().__init__()
+        self.base_layer = base_layer
+        self.hidden_size = hidden_size
+        self.dtype = dtype
+        self.device = device
+
+    @property
+    def vocab_size(self):
+        return self.base_layer.vocab_size
+
+    def __getattr__(self, name):
+        # logits_as_input, scale, org_vocab_size, include_gpu_probs_tensor, ...: the base layer's
+        try:
+            return super().__getattr__(name)
+        except AttributeError:
+            if name == "base_layer":
+                raise
+            return getattr(self.base_layer, name)
+
+    def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
+        self.weight_stacked = torch.zeros((max_deltas, self.base_layer.vocab_size, self.hidden_size),
+                                          dtype=self.dtype, device=self.device)
+        self.indices = None
+        self.indices_padded = None
+        self.indices_len = None
+        self.bitwidth = [0] * max_deltas
+
+    def reset_delta(self, index: int):
+        self.weight_stacked[index] = 0
+        self.bitwidth[index] = 0
+
+    def set_delta(self, index: int, bitwidth: int, weight: torch.Tensor, *unused):
+        self.reset_delta(index)
+        self.bitwidth[index] = bitwidth
+        self.weight_stacked[index, :, :].copy_(weight, non_blocking=ASYNC_COPY)
+
+    def set_mapping(self, base_indices, sampler_indices, sampler_indices_padded=None, embeddings_indices=None,
+                    indices_len: Optional[List[int]] = None):
+        self.indices = sampler_indices
+        self.indices_padded = sampler_indices_padded
+        self.indices_len = indices_len
+
+    def _get_logits(self, hidden_states: torch.Tensor, embedding: torch.Tensor,
+                    embedding_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        return ops.apply_delta_uncompressed(hidden_states, self.weight_stacked,
+                                            self.indices[: self.indices_len[1]], base_embedding=embedding)
+
+    def forward(self, *args, **kwargs):
+        base_forward = getattr(type(self.base_layer), "forward", None)
+        if base_forward is None or base_forward is nn.Module.forward:
+            return self._get_logits(*args, **kwargs)
+        return base_forward(self, *args, **kwargs)
+
+    @classmethod
+    def can_replace_layer(cls, source_layer, delta_config, packed_modules_list, model_config=None) -> bool:
+        return False      # special handling: see from_layer_logits_processor
+
+
+_all_delta_classes = (VocabParallelEmbeddingWithDelta, ColumnParallelLinearWithDelta,
+                      MergedColumnParallelLinearWithDelta,
                       MergedQKVParallelLinearWithDelta, RowParallelLinearWithDelta)
+
+
+def from_layer_logits_processor(layer, lm_head: nn.Module, max_deltas: int, delta_config: DeltaConfig,
+                                model_config=None) -> LogitsProcessorWithDelta:
+    """layers_marlin.py:753-768."""
+    w = lm_head.weight
+    ret = LogitsProcessorWithDelta(layer, w.shape[1], w.dtype, w.device)
+    ret.create_delta_weights(max_deltas, delta_config, model_config)
+    return ret
 
 
 def from_layer(layer: nn.Module, max_deltas: int, delta_config: DeltaConfig, packed_modules_list: List,

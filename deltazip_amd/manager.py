@@ -9,9 +9,10 @@ Mirrors serving/vllm/delta/models.py of eth-easl/deltazip:
 
 The manager owns the index buffers; the layers hold views of them (`set_mapping`), and the kernels
 read them on the device when a layer runs.  `activate_delta` copies a delta's native-layout
-tensors from (pinned) host memory into slot `index` of every wrapped layer on the current stream.
-Uncompressed per-delta weights (embedding / lm_head deltas) are not handled here: a DeltaModel's
-entries for modules the manager did not wrap are ignored.
+tensors from (pinned) host memory into slot `index` of every wrapped layer on the current stream:
+the compressed triples of the linear layers and the uncompressed per-delta tables of the embedding
+and of the output projection (the latter held by the model's `logits_processor` sub-module, when
+it has one).
 """
 from __future__ import annotations
 
@@ -27,7 +28,7 @@ import torch.nn as nn
 from . import ops
 from .checkpoint import DeltaModel
 from .config import DeltaConfig
-from .layers import BaseLayerWithDelta, DeltaMapping, from_layer
+from .layers import BaseLayerWithDelta, DeltaMapping, from_layer, from_layer_logits_processor
 
 
 class LRUCache:
@@ -171,11 +172,13 @@ class DeltaModelManager:
         self._last_mapping = None     # slot numbers may have changed under an unchanged mapping
         for module_name, module in self.modules.items():
             module_delta = delta_model.get_delta(module_name)
-            if module_delta is not None and module_delta._compressed:
+            if module_delta is None:
+                module.reset_delta(index)
+            elif module_delta._compressed:
                 module.set_delta(index, delta_model.bitwidth, module_delta.qweight, module_delta.qzeros,
                                  module_delta.scales, module_delta.g_idx, module_delta.meta)
             else:
-                module.reset_delta(index)
+                module.set_delta(index, delta_model.bitwidth, module_delta.weight)
         return True
 
     def _deactivate_delta(self, delta_id: int) -> None:
@@ -266,14 +269,24 @@ class DeltaModelManager:
         for module_name, module in list(self.model.named_modules()):
             if not self._match_target_modules(module_name):
                 continue
-            if module_name.split(".")[-1] in self.embedding_modules:
-                continue      # per-delta embedding / lm_head weights are uncompressed: not this path
-            packed = self.packed_modules_mapping.get(module_name.split(".")[-1], [])
-            new_module = from_layer(module, self.delta_slots, self.delta_config, packed,
-                                    getattr(self.model, "config", None))
-            if not isinstance(new_module, BaseLayerWithDelta):
-                continue      # embedding / lm_head deltas are not part of this path
-            replace_submodule(self.model, module_name, new_module)
+            last = module_name.split(".")[-1]
+            model_config = getattr(self.model, "config", None)
+            if self.embedding_modules.get(last) == "output_embeddings":
+                # the output projection's delta lives in the logits processor (models.py:467-479)
+                try:
+                    logits_processor = self.model.get_submodule("logits_processor")
+                except AttributeError:
+                    continue
+                new_module = replace_submodule(
+                    self.model, "logits_processor",
+                    from_layer_logits_processor(logits_processor, module, self.delta_slots, self.delta_config,
+                                                model_config))
+            else:
+                packed = self.packed_modules_mapping.get(last, [])
+                new_module = from_layer(module, self.delta_slots, self.delta_config, packed, model_config)
+                if not isinstance(new_module, BaseLayerWithDelta):
+                    continue
+                replace_submodule(self.model, module_name, new_module)
             self.register_module(module_name, new_module)
             self._register_packed_modules(module_name)
             new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,

@@ -127,6 +127,71 @@ def segment(indices: torch.Tensor, num_slots: int):
     return perm, off
 
 
+def apply_delta_embed(x: torch.Tensor, delta_weights: torch.Tensor, indices: torch.Tensor,
+                      base_weight: torch.Tensor) -> torch.Tensor:
+    """Embedding lookup where every token reads the table of its own delta
+    (serving/vllm/delta/deltazip_marlin.py:56-86): out[t] = delta_weights[indices[t]][x[t]], or
+    base_weight[x[t]] for indices[t] == -1.  x [T] int64 token ids, delta_weights [S, V, H] fp16,
+    base_weight [V, H] fp16; returns [T, H] fp16."""
+    _need_cuda(x, delta_weights, indices, base_weight)
+    if x.dtype != torch.int64 or indices.dtype != torch.int64:
+        raise ValueError("token ids and indices must be int64")
+    if delta_weights.dtype != torch.float16 or base_weight.dtype != torch.float16:
+        raise ValueError("embedding tables must be float16")
+    S, V, H = delta_weights.shape
+    if tuple(base_weight.shape) != (V, H) or not delta_weights.is_contiguous() or not base_weight.is_contiguous():
+        raise ValueError("base_weight must be [V, H] like each delta table, all contiguous")
+    T = x.numel()
+    if indices.numel() != T:
+        raise ValueError("one index per token is required")
+    out = torch.empty((T, H), dtype=torch.float16, device=x.device)
+    rc = _lib.lib().dz_embedding_select(x.reshape(-1).contiguous().data_ptr(), indices.contiguous().data_ptr(),
+                                        base_weight.data_ptr(), delta_weights.data_ptr(), V * H, S,
+                                        out.data_ptr(), T, V, H, H, _stream())
+    _lib.check(rc, "dz_embedding_select")
+    return out.view(*x.shape, H)
+
+
+def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indices: torch.Tensor,
+                             base_embedding: torch.Tensor) -> torch.Tensor:
+    """Per-row dense product against the row's own full weight
+    (serving/vllm/delta/deltazip_marlin.py:21-53, the lm_head of LogitsProcessorWithDelta):
+    out[t] = x[t] @ delta_weights[indices[t]]^T, or x[t] @ base_embedding^T for indices[t] == -1.
+    The rows are grouped by id on the device and every group is one set of tiles of the grouped
+    matrix-core GEMM; like the reference's loop over torch.unique(indices), this reads the segment
+    sizes back to the host once."""
+    _need_cuda(x, delta_weights, indices, base_embedding)
+    if x.dtype != torch.float16 or delta_weights.dtype != torch.float16 or base_embedding.dtype != torch.float16:
+        raise ValueError("x and the weights must be float16")
+    S, N, K = delta_weights.shape
+    T = x.shape[0]
+    if x.dim() != 2 or x.shape[1] != K or tuple(base_embedding.shape) != (N, K) or indices.numel() != T:
+        raise ValueError("shapes: x [T, K], delta_weights [S, N, K], base_embedding [N, K], indices [T]")
+    if not (delta_weights.is_contiguous() and base_embedding.is_contiguous()):
+        raise ValueError("weights must be contiguous")
+    perm, seg_off = segment(indices.contiguous(), S)
+    off = seg_off.cpu().tolist()
+    perm64 = perm.long()
+    xs = x.index_select(0, perm64)
+    ys = torch.empty((T, N), dtype=torch.float16, device=x.device)
+    lib, st = _lib.lib(), _stream()
+
+    def launch(w, w2, tiles):
+        tt = torch.tensor(tiles, dtype=torch.int32, device=x.device)
+        _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), w, w2, N * K, tt.data_ptr(), len(tiles), ys.data_ptr(),
+                                           T, K, N, 0, N, st), "dz_gemm_f16_grouped")
+
+    blocks = lambda lo, hi, g: [(r, min(r + 256, hi), g, 0) for r in range(lo, hi, 256)]
+    if off[1] > off[0]:
+        launch(base_embedding.data_ptr(), None, blocks(off[0], off[1], -1))
+    tiles = [b for d in range(S) for b in blocks(off[d + 1], off[d + 2], d)]
+    if tiles:
+        launch(None, delta_weights.data_ptr(), tiles)
+    out = torch.empty_like(ys)
+    out.index_copy_(0, perm64, ys)
+    return out
+
+
 def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_ids: torch.Tensor,
             max_deltas: int, vocab_size: int, extra_vocab_size: int, base_indices: torch.Tensor,
             sampler_indices: Optional[torch.Tensor] = None,

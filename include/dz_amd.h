@@ -99,6 +99,16 @@ int dz_map_ids(const int64_t* token_ids, int T, const int64_t* prompt_ids, int P
                int64_t* base_indices, int64_t* sampler_indices, int64_t* sampler_indices_padded,
                int64_t* embeddings_indices, int ld_emb, int32_t* n_missing, void* stream);
 
+/* Per-token embedding lookup with per-delta tables: out[t, :] = table(t)[tokens[t], :], where
+ * table(t) is weight_stack + indices[t] * stack_stride (elements; a delta's own [V, H] fp16
+ * table) for 0 <= indices[t] < S and base_weight [V, H] otherwise.  The fine-tuned table replaces
+ * the base one, it is not added: apply_delta_embed, serving/vllm/delta/deltazip_marlin.py:56-86,
+ * as called by VocabParallelEmbeddingWithDelta.forward, layers_marlin.py:143-160.  A token id
+ * outside [0, V) gives a row of zeros.  H % 8 == 0, ldo % 8 == 0 (row stride of out, elements). */
+int dz_embedding_select(const int64_t* tokens, const int64_t* indices, const uint16_t* base_weight,
+                        const uint16_t* weight_stack, long long stack_stride, int S, uint16_t* out, int T,
+                        int V, int H, int ldo, void* stream);
+
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
  * zero-filled once before first use; calls leave it ready for the next call.  Calls that share
  * a workspace must be ordered on one stream. */

@@ -16,6 +16,8 @@ Pinning status (what independent evidence each function is checked against in te
   native layout functions       defined by this project; pinned by round trip through
                                 dequant_gptq
   convert_mapping_ref           hand-computed index tensors for small batches          (pinned)
+  embed_select_ref, linear_select_ref   plain row selection / torch CPU matmul per row, checked
+                                against hand-built tables                              (pinned)
 The fused third-party kernel the reference calls on the serving path (triteia
 `sbmm_4bit_2_4_native`, un-vendored and un-pinned: scripts/install.sh:2, call site
 serving/vllm/delta/deltazip_marlin.py:18) cannot be inspected: its bit layout and rounding are
@@ -421,6 +423,32 @@ def convert_mapping_ref(index_mapping, prompt_mapping, delta_index_to_id, max_de
     padded[padded == -1] = max_deltas - 1
     padded = np.arange(len(padded), dtype=np.int64) + padded * len(padded)
     return base, sampler, padded, emb2
+
+
+# --------------------------------------------------------------------------------------
+# uncompressed per-delta tables: embedding and output projection
+# (serving/vllm/delta/deltazip_marlin.py:21-86)
+# --------------------------------------------------------------------------------------
+
+
+def embed_select_ref(tokens, delta_weights, ids, base_weight) -> np.ndarray:
+    """deltazip_marlin.py:56-86: row tokens[t] of delta_weights[ids[t]], or of base_weight for
+    ids[t] == -1 (the delta's table replaces the base table)."""
+    out = np.zeros((len(tokens), base_weight.shape[1]), dtype=base_weight.dtype)
+    for t, (tok, d) in enumerate(zip(tokens, ids)):
+        out[t] = (base_weight if d == -1 else delta_weights[int(d)])[int(tok)]
+    return out
+
+
+def linear_select_ref(x16, delta_weights, ids, base_weight) -> np.ndarray:
+    """deltazip_marlin.py:21-53: F.linear(x[t], W) with W = delta_weights[ids[t]] or base_weight
+    for ids[t] == -1; fp32 result [T, N]."""
+    x = torch.from_numpy(np.ascontiguousarray(x16).astype(np.float32))
+    out = np.zeros((x.shape[0], base_weight.shape[0]), dtype=np.float32)
+    for t, d in enumerate(ids):
+        w = base_weight if d == -1 else delta_weights[int(d)]
+        out[t] = (torch.from_numpy(np.ascontiguousarray(w).astype(np.float32)) @ x[t]).numpy()
+    return out
 
 
 # --------------------------------------------------------------------------------------

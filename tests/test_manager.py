@@ -10,7 +10,8 @@ from oracle import dz_oracle as o
 from deltazip_amd import (DeltaConfig, DeltaMapping, DeltaModel, CompressionConfig, LRUCacheDeltaModelManager,
                           DeltaModelManager, create_delta_manager, convert_model)
 from deltazip_amd.layers import (MergedQKVParallelLinearWithDelta, MergedColumnParallelLinearWithDelta,
-                                 RowParallelLinearWithDelta)
+                                 RowParallelLinearWithDelta, VocabParallelEmbeddingWithDelta,
+                                 LogitsProcessorWithDelta)
 from deltazip_amd.manager import LRUCache
 
 H, I, V = 256, 512, 64
@@ -43,6 +44,22 @@ class Inner(nn.Module):
         self.layers = nn.ModuleList([Block(dev) for _ in range(layers)])
 
 
+class ToyLogitsProcessor(nn.Module):
+    """The serving engine's LogitsProcessor reduced to what the delta wrapper uses: `vocab_size`
+    and a forward that calls `_get_logits(hidden_states, embedding, embedding_bias)`."""
+
+    def __init__(self, vocab_size):
+        super().__init__()
+        self.vocab_size = vocab_size
+        self.scale = 1.0
+
+    def _get_logits(self, hidden_states, embedding, embedding_bias=None):
+        return hidden_states @ embedding.t()
+
+    def forward(self, embedding, hidden_states):
+        return self._get_logits(hidden_states, embedding, None) * self.scale
+
+
 class ToyModel(nn.Module):
     """Module tree and class attributes shaped like the serving model
     (model_executor/models/llama.py:299-340)."""
@@ -53,6 +70,7 @@ class ToyModel(nn.Module):
         super().__init__()
         self.model = Inner(dev, layers)
         self.lm_head = nn.Linear(H, V, bias=False, dtype=torch.float16, device=dev)
+        self.logits_processor = ToyLogitsProcessor(V)
         with torch.no_grad():
             g = torch.Generator().manual_seed(5)
             for p in self.parameters():
@@ -76,6 +94,12 @@ def make_delta_model(delta_id, bits, seed):
              "self_attn.o_proj": ref["self_attn.o_proj"],
              "mlp.gate_up_proj": np.concatenate([ref["mlp.gate_proj"], ref["mlp.up_proj"]], axis=1),
              "mlp.down_proj": ref["mlp.down_proj"]}
+    g = torch.Generator().manual_seed(seed + 77)
+    sd["model.embed_tokens.weight"] = (torch.randn(V, H, generator=g) * 0.02).half()
+    sd["lm_head.weight"] = (torch.randn(V, H, generator=g) * 0.02).half()
+    sd["model.norm.weight"] = torch.ones(H, dtype=torch.float16)
+    fused["model.embed_tokens"] = sd["model.embed_tokens.weight"].numpy()
+    fused["lm_head"] = sd["lm_head.weight"].numpy()
     dm = DeltaModel.from_tensors(sd, delta_id, CompressionConfig(bits=bits, prunen=2, prunem=4, sparsity=0.5),
                                  pin_memory=False)
     return dm, fused
@@ -93,6 +117,18 @@ def test_oracle_convert_mapping_known_answers():
     assert emb.tolist() == [[20, 20, 0, 0, 0], [220, 220, 0, 0, 0]]
     with pytest.raises(ValueError):
         o.convert_mapping_ref((5,), (), [7, None, 3], 4, 100, 0)
+
+
+def test_oracle_table_selection_known_answers():
+    base = np.arange(12, dtype=np.float16).reshape(4, 3)                 # row r = [3r, 3r+1, 3r+2]
+    stack = np.stack([base + 100, base + 200]).astype(np.float16)
+    got = o.embed_select_ref([3, 0, 2], stack, [-1, 1, 0], base)
+    assert got.tolist() == [[9, 10, 11], [200, 201, 202], [106, 107, 108]]
+    x = np.array([[1, 0, 0], [0, 1, 0], [1, 1, 1]], dtype=np.float16)
+    y = o.linear_select_ref(x, stack, [0, -1, 1], base)
+    assert y[0].tolist() == [100, 103, 106, 109]         # column 0 of table 0
+    assert y[1].tolist() == [1, 4, 7, 10]                # column 1 of the base table
+    assert y[2].tolist() == [603, 612, 621, 630]         # row sums of table 1
 
 
 def test_lru_cache_order_and_callbacks():
@@ -117,9 +153,12 @@ def test_manager_wraps_modules_and_tracks_slots(dzlib):
     assert isinstance(model.model.layers[0].self_attn.qkv_proj, MergedQKVParallelLinearWithDelta)
     assert isinstance(model.model.layers[0].mlp.gate_up_proj, MergedColumnParallelLinearWithDelta)
     assert isinstance(model.model.layers[0].mlp.down_proj, RowParallelLinearWithDelta)
-    assert isinstance(model.model.embed_tokens, nn.Embedding)         # not wrapped: outside this path
-    assert sorted(mgr.modules) == ["model.layers.0.mlp.down_proj", "model.layers.0.mlp.gate_up_proj",
-                                   "model.layers.0.self_attn.o_proj", "model.layers.0.self_attn.qkv_proj"]
+    assert isinstance(model.model.embed_tokens, VocabParallelEmbeddingWithDelta)
+    assert isinstance(model.logits_processor, LogitsProcessorWithDelta) and isinstance(model.lm_head, nn.Linear)
+    assert mgr.modules["lm_head"] is model.logits_processor and model.logits_processor.scale == 1.0
+    assert sorted(mgr.modules) == ["lm_head", "model.embed_tokens", "model.layers.0.mlp.down_proj",
+                                   "model.layers.0.mlp.gate_up_proj", "model.layers.0.self_attn.o_proj",
+                                   "model.layers.0.self_attn.qkv_proj"]
     assert mgr.packed_modules["model.layers.0.self_attn.qkv_proj"] == [
         "model.layers.0.self_attn.q_proj", "model.layers.0.self_attn.k_proj", "model.layers.0.self_attn.v_proj"]
     qkv = model.model.layers[0].self_attn.qkv_proj
@@ -139,6 +178,8 @@ def test_manager_wraps_modules_and_tracks_slots(dzlib):
     want = dms[1].get_delta("model.layers.0.self_attn.qkv_proj")
     assert torch.equal(qkv.qweight_stacked[0].reshape(-1), want.qweight.reshape(-1))
     assert torch.equal(qkv.scales_stacked[0].reshape(-1), want.scales.reshape(-1))
+    assert torch.equal(model.model.embed_tokens.delta_weights[0], dms[1].get_delta("model.embed_tokens").weight)
+    assert torch.equal(model.logits_processor.weight_stacked[1], dms[0].get_delta("lm_head").weight)
     assert mgr.deactivate_delta(2) and not mgr.deactivate_delta(2)
     assert mgr.delta_index_to_id == [None, 1]
     assert mgr.activate_delta(3) and mgr.delta_index_to_id == [3, 1]
@@ -214,11 +255,56 @@ def test_map_ids_matches_reference_loop(dev, T, P, S):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("T,S,V_,H_", [(1, 1, 64, 256), (37, 5, 1000, 264), (300, 9, 512, 4096)])
+def test_embedding_select_is_exact(dev, T, S, V_, H_):
+    from deltazip_amd import ops
+    rng = np.random.default_rng(T)
+    base = rng.standard_normal((V_, H_)).astype(np.float16)
+    stack = rng.standard_normal((S, V_, H_)).astype(np.float16)
+    tok = rng.integers(0, V_, size=T)
+    ids = rng.integers(-1, S, size=T)
+    got = ops.apply_delta_embed(torch.from_numpy(tok).to(dev), torch.from_numpy(stack).to(dev),
+                                torch.from_numpy(ids).to(dev), torch.from_numpy(base).to(dev))
+    torch.cuda.synchronize()
+    want = o.embed_select_ref(tok, stack, ids, base)
+    assert got.dtype == torch.float16 and np.array_equal(got.cpu().numpy().view(np.uint16), want.view(np.uint16))
+    # a token id outside the vocabulary gives zeros, ids outside [0, S) read the base table
+    got = ops.apply_delta_embed(torch.tensor([V_, 1], device=dev), torch.from_numpy(stack).to(dev),
+                                torch.tensor([0, S + 3], device=dev), torch.from_numpy(base).to(dev))
+    assert (got[0] == 0).all() and np.array_equal(got[1].cpu().numpy(), base[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("T,S,N,K", [(1, 1, 64, 256), (32, 8, 1000, 512), (128, 3, 32000, 256), (300, 4, 512, 320)])
+def test_uncompressed_projection_matches_loop(dev, T, S, N, K):
+    from deltazip_amd import ops
+    rng = np.random.default_rng(T + N)
+    base = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    stack = (rng.standard_normal((S, N, K)) * 0.05).astype(np.float16)
+    x = rng.standard_normal((T, K)).astype(np.float16)
+    ids = rng.integers(-1, S, size=T)
+    if T > 2:
+        ids[0], ids[1] = -1, S - 1
+    got = ops.apply_delta_uncompressed(torch.from_numpy(x).to(dev), torch.from_numpy(stack).to(dev),
+                                       torch.from_numpy(ids).to(dev), torch.from_numpy(base).to(dev))
+    torch.cuda.synchronize()
+    want = o.linear_select_ref(x, stack, ids, base)
+    assert tuple(got.shape) == (T, N) and o.rel_err(got.float().cpu().numpy(), want) <= 1e-2
+    # all rows on the base weight: the plain product
+    got = ops.apply_delta_uncompressed(torch.from_numpy(x).to(dev), torch.from_numpy(stack).to(dev),
+                                       torch.full((T,), -1, dtype=torch.long, device=dev),
+                                       torch.from_numpy(base).to(dev))
+    ref = x.astype(np.float32) @ base.astype(np.float32).T
+    assert o.rel_err(got.float().cpu().numpy(), ref) <= 1e-2
+
+
+@pytest.mark.gpu
 def test_checkpoint_to_manager_to_forward(dev):
     bits = 4
     model = ToyModel(dev)
     base = {n: m.weight.detach().cpu().numpy().copy() for n, m in model.named_modules()
             if isinstance(m, nn.Linear)}
+    base_emb = model.model.embed_tokens.weight.detach().cpu().numpy().copy()
     mgr = create_delta_manager(model, 8, 64, V, DeltaConfig(max_deltas=3, max_bitwidth=bits, max_cpu_deltas=4),
                                delta_manager_cls=LRUCacheDeltaModelManager)
     fused = {}
@@ -245,6 +331,17 @@ def test_checkpoint_to_manager_to_forward(dev):
             ref = o.forward_ref(x.cpu().numpy(), base["model.layers.0." + name], [table[i] for i in uniq],
                                 np.array([uniq.index(i) if i > 0 else -1 for i in ids]))
             assert bias is None and o.rel_err(y.float().cpu().numpy(), ref) <= 1e-2, name
+        # embedding and output projection: the delta's own tables
+        slots_np = np.array(slots)
+        tok = np.arange(len(ids)) % V
+        by_slot = lambda name: np.stack([fused[d][name] if d is not None else np.zeros((V, H), np.float16)
+                                         for d in mgr.delta_index_to_id])
+        e = model.model.embed_tokens(torch.from_numpy(tok).to(dev))
+        assert np.array_equal(e.cpu().numpy(), o.embed_select_ref(tok, by_slot("model.embed_tokens"), slots_np,
+                                                                  base_emb))
+        logits = model.logits_processor(model.lm_head.weight, x[:2])
+        want = o.linear_select_ref(x[:2].cpu().numpy(), by_slot("lm_head"), slots_np[:2], base["lm_head"])
+        assert o.rel_err(logits.float().cpu().numpy(), want) <= 1e-2
 
     check(ids)
     # delta 14 takes the least recently used slot (12's: 11 and 13 were activated after it)
