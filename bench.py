@@ -277,7 +277,7 @@ def main():
         achieved = (step_flops / len(shapes)) / avg_launch_s / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
-                    "kernel": "dz_gemm_kernel (pair)", "algorithmic_flops_per_call": step_flops / len(shapes),
+                    "kernel": "dz_gemm24_kernel", "algorithmic_flops_per_call": step_flops / len(shapes),
                     "avg_call_us": round(avg_launch_s * 1e6, 2)}
 
     out = {

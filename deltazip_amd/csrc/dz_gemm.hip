@@ -180,9 +180,9 @@ int gemm_launch(GemmParams P, int ntiles_m, void* stream) {
   if (((uintptr_t)P.x & 15) || ((uintptr_t)P.w & 15) || ((uintptr_t)P.w2 & 15) || ((uintptr_t)P.y & 7) ||
       (P.w2 && (P.w2_stride & 7)))
     return DZ_EALIGN;
-  if ((unsigned long long)P.T * (unsigned)P.K * 2ull >= (1ull << 32) ||
-      (unsigned long long)P.N * (unsigned)P.K * 2ull >= (1ull << 32))
-    return DZ_ESHAPE;   // 32-bit row offsets inside one operand
+  if ((unsigned long long)P.T * (unsigned)P.K * 2ull >= (1ull << 31) ||
+      (unsigned long long)P.N * (unsigned)P.K * 2ull >= (1ull << 31))
+    return DZ_ESHAPE;   // byte offsets inside one operand stay below 2^31 (buffer addressing)
   P.tiles_m = ntiles_m;
   P.tiles_n = (P.N + BN - 1) / BN;
   const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;

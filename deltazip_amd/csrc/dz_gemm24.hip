@@ -1,0 +1,350 @@
+// Prefill-sized multi-delta linear layer on the gfx950 matrix cores, deltas taken in packed form:
+//   y[t, :] (+)= x[t, :] @ w_base^T + x[t, :] @ dequant(delta[slot(t)])^T
+// for tokens grouped by delta slot (a table of row blocks, each with one slot).
+//
+// One workgroup (8 wavefronts, two per SIMD) computes 256 output features x 256 tokens of one row
+// block; each wavefront owns 128 features x 64 tokens as 8 x 4 tiles of 16 x 16 (128 fp32
+// accumulators, in ordinary vector registers: the sparse instruction does not accumulate in the
+// accumulation registers).  K is walked
+// twice in slabs of 64 columns, into the same accumulators:
+//   base pass   weight slab and activation slab go from global memory straight into LDS (two
+//               buffers, the next slab is on its way while this one is multiplied);
+//               v_mfma_f32_16x16x32_f16.
+//   delta pass  the activation slab goes through LDS as before; the delta's packed codes and 2-bit
+//               positions (native layout: 16 bytes per lane per 32 x 256 tile, already in operand
+//               order) are staged one k-block ahead in the idle weight half of the LDS buffers,
+//               read back 16 bytes per lane, unpacked to fp16(scale * (q - zero)) -- the
+//               reference's rounding point, qlinear_cuda.py:306-308 -- and fed to the 2:4-sparse
+//               v_smfmac_f32_16x16x64_f16 together with their positions: half the matrix-core time
+//               of a dense product, and no dequantised copy of the delta ever exists in memory.
+// Rows of x and y are addressed through an optional token order (the output of the segment sort),
+// so the batch is neither gathered nor scattered.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/dz_amd.h"
+#include "dz_device.h"
+
+namespace {
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int SLAB = 256 * BK * 2;        // bytes of one operand slab in LDS
+constexpr int GM = 4, GN = 8;             // tiles per XCD block
+
+struct Gemm24Params {
+  const _Float16* x;
+  const _Float16* w;             // base weight [N, K] or nullptr
+  const u4_t* codes;
+  const u4_t* meta;
+  const _Float16* scales;
+  long long codes_slot_u4, meta_slot_u4, scales_slot;
+  const dz_gemm_tile* tiles;     // row blocks (device memory)
+  const int* perm;               // token order or nullptr
+  _Float16* y;
+  int T, K, N, S, G, gslabs, accumulate, ldy, tiles_m, tiles_n, NKB, NP;   // gslabs: slabs per scale group
+};
+
+template <int BITS>
+__global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2 buffers][w slab | x slab]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wn = wave & 1, wq = wave >> 1;       // feature half (128), token quarter (64)
+  const int li = lane & 15, lg = lane >> 4;
+  const uint32_t MAGIC = magic_vgpr();
+
+  // workgroup -> tile: XCD-local blocks of GM x GN tiles
+  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+  const int sbn = (P.tiles_n + GN - 1) / GN;
+  const int sb = (q / (GM * GN)) * 8 + xcd, r = q % (GM * GN);
+  const int tm = (sb / sbn) * GM + r / GN, tn = (sb % sbn) * GN + r % GN;
+  if (tm >= P.tiles_m || tn >= P.tiles_n) return;
+  const int row_lo = P.tiles[tm].row_lo, row_hi = P.tiles[tm].row_hi, slot = P.tiles[tm].group;
+  if (row_hi <= row_lo) return;                  // unused entry of the table
+  const int n0 = tn * BN;
+  const bool has_delta = slot >= 0 && slot < P.S;
+  const int nslab1 = P.K / BK;
+  const int nb = P.w ? nslab1 : 0, nd = has_delta ? nslab1 : 0, total = nb + nd;
+  const unsigned Kb = (unsigned)P.K * 2u;
+  // a wavefront whose 64 token rows lie beyond the block only helps with the loads
+  const bool has_rows = row_lo + wq * 64 < row_hi;
+
+  f4_t acc[8][4];
+#pragma unroll
+  for (int a = 0; a < 8; ++a)
+#pragma unroll
+    for (int b = 0; b < 4; ++b) acc[a][b] = (f4_t){0.f, 0.f, 0.f, 0.f};
+
+  // ---- slab loader.  A slab is 32 requests of 1 KiB (8 rows x 128 bytes); every wavefront issues 4
+  // of the weight slab and 4 of the activation slab.  Lane l fills LDS row l/8, physical chunk l%8
+  // with global chunk (l%8) ^ ((row >> 1) & 7): a 16-byte read is served 16 lanes per cycle, and
+  // 16 consecutive rows then fall on 16 different bank groups.
+  const int lr = lane >> 3;
+  unsigned goff_w[4], goff_x[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int R = (wave * 4 + i) * 8 + lr;
+    const int lc = (lane & 7) ^ ((R >> 1) & 7);
+    goff_w[i] = (unsigned)min(n0 + R, P.N - 1) * Kb + (unsigned)lc * 16u;     // clamped rows: never stored
+    const int pos = min(row_lo + R, row_hi - 1);
+    const int row = P.perm ? P.perm[pos] : pos;
+    goff_x[i] = (unsigned)row * Kb + (unsigned)lc * 16u;
+  }
+  const __amdgpu_buffer_rsrc_t rw =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.w ? P.w : P.x), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rx =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.x), 0, 0x7fffffff, 0x00020000);
+  auto issue = [&](int s, int buf) {
+    const bool base = s < nb;
+    const int soff = (base ? s : s - nb) * (BK * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      unsigned char* dst = smem + buf * (2 * SLAB) + (wave * 4 + i) * 1024;
+      if (base)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 (int)goff_w[i], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(dst + SLAB), 16,
+                                               (int)goff_x[i], soff, 0, 0);
+    }
+  };
+
+  // ---- packed delta operands: the 8 n-pairs (256 rows) of the workgroup's tile, one k-block at a
+  // time, staged in the weight half of an LDS buffer (idle during the delta pass): wavefront w
+  // fetches n-pair w -- 1 KiB of positions and 1 or 2 KiB of codes, already in lane order -- and
+  // every wavefront later reads the four n-pairs of its own feature half from there.
+  constexpr int DT = (BITS == 2) ? 2048 : 3072;          // staged bytes per n-pair
+  auto issue_delta = [&](int kb) {
+    unsigned char* dst = smem + (kb & 1) * (2 * SLAB) + wave * DT;
+    const int np = min(n0 / DZ_NPAIR + wave, P.NP - 1);
+    const size_t tile = (size_t)np * P.NKB + kb;
+    const char* mb = (const char*)(P.meta + (size_t)slot * P.meta_slot_u4 + tile * 64) + lane * 16;
+    const char* cb = (const char*)(P.codes + (size_t)slot * P.codes_slot_u4 + tile * (BITS == 2 ? 64 : 128)) + lane * 16;
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)mb,
+                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)cb,
+                                     (__attribute__((address_space(3))) void*)(dst + 1024), 16, 0, 0);
+    if (BITS == 4)
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(cb + 1024),
+                                       (__attribute__((address_space(3))) void*)(dst + 2048), 16, 0, 0);
+  };
+  // scales of scale group gi for the lane's 8 operand rows: row n0 + wn*128 + 16*t + i
+  // (two per register: entry p holds the scales of the two 16-row halves of n-pair p)
+  auto load_scales = [&](h2_t (&sc)[4], int gi) {
+    const _Float16* sp = P.scales + (size_t)slot * P.scales_slot + (size_t)min(gi, P.G - 1) * P.N;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      sc[p][0] = sp[min(n0 + wn * 128 + 32 * p + li, P.N - 1)];
+      sc[p][1] = sp[min(n0 + wn * 128 + 32 * p + 16 + li, P.N - 1)];
+    }
+  };
+
+  // ---- operand addresses: lane (i = lane % 16, g = lane / 16) reads row i of a 16-row tile, chunk
+  // 4*h + g of the slab row (columns 32*h + 8*g ..): the dense operand order of two 16x16x32
+  // products, and the order the sparse product expects of its dense operand
+  int foff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) foff[h] = (((4 * h + lg) ^ ((li >> 1) & 7)) << 4);
+  const int wrow = (wn * 128 + li) * 128, xrow = (wq * 64 + li) * 128;
+
+  if (total > 0) issue(0, 0);
+  if (nb == 0 && nd > 0) issue_delta(0);
+  // ---- base pass
+  for (int s = 0; s < nb; ++s) {
+    const int buf = s & 1;
+    // the slab of this turn was requested one turn ago: wait for this wavefront's share, then meet
+    // the others (their shares are in, and nobody still reads the buffer filled next)
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
+    __syncthreads();
+    if (s + 1 < total) issue(s + 1, buf ^ 1);
+    // the last base slab sits in buffer 1 (the slab count is a multiple of 4): the weight half of
+    // buffer 0 is free for the first k-block of the delta
+    if (s + 1 == nb && nd > 0) issue_delta(0);
+    if (!has_rows) continue;
+    const unsigned char* wb = smem + buf * (2 * SLAB);
+    const unsigned char* xb = wb + SLAB;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      h8_t fw[8], fx[4];
+#pragma unroll
+      for (int a = 0; a < 8; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[h]);
+#pragma unroll
+      for (int b = 0; b < 4; ++b)
+#pragma unroll
+        for (int a = 0; a < 8; ++a)
+          acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[a], fx[b], acc[a][b], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);   // one half-slab's operands at a time
+    }
+  }
+  // ---- delta pass
+  Frag<BITS> cur[4];
+  h2_t sc[4], scn[4];
+  if (nd > 0) load_scales(scn, 0);
+  int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
+  for (int sd = 0; sd < nd; ++sd) {
+    const int s = nb + sd, buf = s & 1;
+    const int kb = sd >> 2, j = sd & 3;
+    __builtin_amdgcn_s_waitcnt(0x0070);
+    __syncthreads();
+    if (s + 1 < total) issue(s + 1, buf ^ 1);
+    if (j == 0) {
+      // this k-block's packed operands were staged a k-block ago; the other staging area is free
+      // (every wavefront has passed the barrier above, so nobody reads it any more)
+      const unsigned char* dsrc = smem + (kb & 1) * (2 * SLAB) + (wn * 4) * DT + lane * 16;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        cur[p].meta = *(const u4_t*)(dsrc + p * DT);
+        cur[p].code[0] = *(const u4_t*)(dsrc + p * DT + 1024);
+        if (BITS == 4) cur[p].code[BITS == 2 ? 0 : 1] = *(const u4_t*)(dsrc + p * DT + 2048);
+      }
+      if (kb + 1 < P.NKB) issue_delta(kb + 1);
+    }
+    // scales: a scale group spans whole slabs (group size is a multiple of 64); the next group's
+    // scales are requested during the last slab of the current one
+    if (gleft == P.gslabs) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) sc[t] = scn[t];
+    }
+    if (gleft == 1 && sd + 1 < nd) load_scales(scn, gi + 1);
+    if (--gleft == 0) {
+      gleft = P.gslabs;
+      ++gi;
+    }
+    if (!has_rows) continue;
+    const unsigned char* xb = smem + buf * (2 * SLAB) + SLAB;
+    h16_t B[4];
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const h8_t lo = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[0]);
+      const h8_t hi = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[1]);
+      B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      // word j of the lane's four words; a compile-time index after unrolling over the four cases
+      uint32_t cw0 = 0, cw1 = 0, mw = 0;
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        if (jj == j) {
+          mw = cur[p].meta[jj];
+          if (BITS == 2) {
+            cw0 = cur[p].code[0][jj];
+          } else {
+            cw0 = cur[p].code[BITS == 2 ? 0 : (jj >> 1)][2 * (jj & 1) + 0];
+            cw1 = cur[p].code[BITS == 2 ? 0 : (jj >> 1)][2 * (jj & 1) + 1];
+          }
+        }
+      }
+      h8_t A0, A1;
+      if (BITS == 2) {
+        unpack2(cw0, MAGIC, A0, A1);
+      } else {
+        A0 = unpack4(cw0, MAGIC);
+        A1 = unpack4(cw1, MAGIC);
+      }
+      A0 *= sc[p][0];
+      A1 *= sc[p][1];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        acc[2 * p][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B[b], acc[2 * p][b], (int)mw, 0, 0);
+        acc[2 * p + 1][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B[b], acc[2 * p + 1][b], (int)mw, 0, 1);
+      }
+    }
+  }
+
+  // ---- store: lane (i, g) holds features 4*g .. 4*g + 3 of tile a for token i of tile b
+#pragma unroll
+  for (int b = 0; b < 4; ++b) {
+    const int pos = row_lo + wq * 64 + b * 16 + li;
+    if (pos >= row_hi) continue;
+    const int row = P.perm ? P.perm[pos] : pos;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const int n = n0 + wn * 128 + a * 16 + 4 * lg;
+      if (n >= P.N) continue;
+      f4_t v = acc[a][b];
+      _Float16* yp = P.y + (size_t)row * P.ldy + n;
+      if (P.accumulate) {
+        const h4_t o = *(const h4_t*)yp;
+        v += (f4_t){(float)o[0], (float)o[1], (float)o[2], (float)o[3]};
+      }
+      const h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+      *(h4_t*)yp = o;
+    }
+  }
+}
+
+// Row blocks from segment offsets: segment k (k = 0: tokens without a delta, k >= 1: slot k - 1)
+// is cut into blocks of at most 256 rows; unused entries of the table are left empty.
+__global__ __launch_bounds__(1024) void dz_build_tiles_kernel(const int* __restrict__ seg_off, int S,
+                                                              dz_gemm_tile* __restrict__ tiles, int max_tiles) {
+  extern __shared__ int first[];    // first[k]: index of segment k's first block; first[S + 1]: total
+  const int tid = threadIdx.x, nseg = S + 1;
+  for (int k = tid; k < nseg; k += 1024) first[k + 1] = (seg_off[k + 1] - seg_off[k] + BM - 1) / BM;
+  if (tid == 0) first[0] = 0;
+  __syncthreads();
+  if (tid == 0)
+    for (int k = 1; k <= nseg; ++k) first[k] += first[k - 1];
+  __syncthreads();
+  for (int k = tid; k < nseg; k += 1024) {
+    const int lo = seg_off[k], hi = seg_off[k + 1];
+    for (int t = first[k], r = lo; r < hi && t < max_tiles; ++t, r += BM)
+      tiles[t] = dz_gemm_tile{r, min(r + BM, hi), k - 1, 0};
+  }
+  for (int t = first[nseg] + tid; t < max_tiles; t += 1024) tiles[t] = dz_gemm_tile{0, 0, -1, 0};
+}
+
+}  // namespace
+
+extern "C" int dz_build_tiles(const int32_t* seg_off, int S, dz_gemm_tile* tiles, int max_tiles, void* stream) {
+  if (!seg_off || !tiles) return DZ_EINVAL;
+  if (S < 0 || S > DZ_MAX_SLOTS_SEGMENT || max_tiles < 1) return DZ_ESHAPE;
+  hipLaunchKernelGGL(dz_build_tiles_kernel, dim3(1), dim3(1024), (size_t)(S + 2) * 4, (hipStream_t)stream,
+                     seg_off, S, tiles, max_tiles);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
+                                   const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                                   int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                                   uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
+  if (!x || !y || !tiles || ntiles < 1 || S < 0) return DZ_EINVAL;
+  if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
+  size_t cb, mb, sb;
+  int rc = dz_native_sizes(K, N, bits, group_size, &cb, &mb, &sb);
+  if (rc) return rc;
+  const int gs = (group_size == -1 || group_size == K) ? K : group_size;
+  if (T < 1 || ldy < N || ldy % 4) return DZ_ESHAPE;
+  if (((uintptr_t)x & 15) || ((uintptr_t)w_base & 15) || ((uintptr_t)y & 7)) return DZ_EALIGN;
+  if ((unsigned long long)T * (unsigned)K * 2ull >= (1ull << 31) ||
+      (unsigned long long)N * (unsigned)K * 2ull >= (1ull << 31))
+    return DZ_ESHAPE;   // byte offsets inside one operand stay below 2^31 (buffer addressing)
+  Gemm24Params P{};
+  P.x = (const _Float16*)x; P.w = (const _Float16*)w_base; P.y = (_Float16*)y;
+  P.codes = (const u4_t*)codes_stacked; P.meta = (const u4_t*)meta_stacked;
+  P.scales = (const _Float16*)scales_stacked;
+  P.codes_slot_u4 = (long long)(cb / 16); P.meta_slot_u4 = (long long)(mb / 16); P.scales_slot = (long long)(sb / 2);
+  P.tiles = tiles; P.perm = perm;
+  P.T = T; P.K = K; P.N = N; P.S = S; P.gslabs = gs / BK; P.G = K / gs; P.accumulate = accumulate; P.ldy = ldy;
+  P.NKB = K / DZ_KBLOCK; P.NP = N / DZ_NPAIR;
+  P.tiles_m = ntiles;
+  P.tiles_n = (N + BN - 1) / BN;
+  const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
+  const int nsb = (sbm * sbn + 7) / 8 * 8;
+  const unsigned grid = (unsigned)nsb * GM * GN;
+  const size_t lds = 2 * 2 * SLAB;
+  static bool attr_done[2] = {false, false};
+  auto go = [&](auto kern, int which) -> int {
+    if (!attr_done[which]) {
+      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return DZ_ELAUNCH;
+      attr_done[which] = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, (hipStream_t)stream, P);
+    return DZ_OK;
+  };
+  rc = bits == 2 ? go(dz_gemm24_kernel<2>, 0) : go(dz_gemm24_kernel<4>, 1);
+  if (rc) return rc;
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}

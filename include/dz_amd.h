@@ -159,6 +159,28 @@ int dz_gemm_f16_grouped(const uint16_t* x, const uint16_t* w, const uint16_t* w2
                         long long w2_stride, const dz_gemm_tile* tiles, int ntiles, uint16_t* y,
                         int T, int K, int N, int accumulate, int ldy, void* stream);
 
+/* Row blocks for dz_multi_delta_gemm from the segment offsets dz_segment wrote (device memory,
+ * S + 2 entries): every segment is cut into blocks of at most 256 rows, group = slot (-1 for the
+ * tokens without a delta); entries of `tiles` (device memory, max_tiles of them) beyond the blocks
+ * in use are marked empty.  max_tiles >= (T + 255) / 256 + min(S + 1, T) always suffices, so the
+ * host never needs to read the offsets back.  S <= DZ_MAX_SLOTS_SEGMENT. */
+int dz_build_tiles(const int32_t* seg_off, int S, dz_gemm_tile* tiles, int max_tiles, void* stream);
+
+/* The layer at prefill sizes, deltas in packed form: for every row block b of `tiles` and every
+ * position p in [row_lo, row_hi), with t = perm ? perm[p] : p,
+ *   y[t, 0..N) (+)= x[t] @ w_base^T + x[t] @ dequant(delta[group(b)])^T
+ * (w_base may be NULL; group -1 or >= S: base only).  Base product on the dense matrix-core
+ * instructions, delta product on the 2:4-sparse ones straight from the native layout; both in the
+ * same fp32 accumulators, every delta value rounded to fp16 exactly as dz_dequant rounds it.
+ * Stands in, like dz_multi_delta_linear, for sbmm_4bit_2_4_native at
+ * serving/vllm/delta/deltazip_marlin.py:18, and for the exllama path's "reconstruct, then dense
+ * GEMM" above 50 rows (q_gemm.cu:118-137) without the reconstruction.  Rows outside every block
+ * are not written.  K % 256 == 0, N % 32 == 0, T * K and N * K below 2^31 elements. */
+int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
+                        const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                        int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                        uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
+
 /* Tuning hook used by the benchmark: override the split of K across workgroups of the fused
  * kernel (0 = automatic). */
 void dz_set_ksplit(int nsplit);

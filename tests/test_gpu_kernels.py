@@ -283,3 +283,55 @@ def test_unsorted_batches_above_32_tokens(dev, t):
     ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
     assert o.rel_err(y, ref) <= TOL
     assert ops.workspace_status() == 0
+
+
+PREFILL_CASES = [
+    # n, k, bits, gs, deltas, tokens, ids
+    (256, 1024, 2, -1, 4, 400, "uniform"),
+    (352, 768, 4, -1, 3, 129, "uniform"),
+    (352, 768, 2, 128, 5, 700, "zipf"),
+    (512, 512, 4, 64, 2, 300, "blocks"),
+    (96, 256, 2, -1, 9, 1000, "uniform"),
+    (288, 1280, 4, 256, 6, 515, "uniform"),
+]
+
+
+@pytest.mark.parametrize("n,k,bits,gs,nd,t,kind", PREFILL_CASES)
+def test_packed_delta_gemm_parity(dev, n, k, bits, gs, nd, t, kind):
+    """T > 128 through dz_segment + dz_build_tiles + dz_multi_delta_gemm: unsorted ids, tokens
+    without a delta, N that is not a multiple of the 256-wide tile, grouped scales, then the
+    delta-only and accumulate forms."""
+    p = make_problem(n, k, bits, gs, nd, t, kind, 4000 + n + k + t, dev)
+    p["ids_np"][::7] = -1
+    p["ids"] = torch.from_numpy(p["ids_np"]).to(dev)
+    y = run_layer(p)
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+    # delta only, accumulated onto an existing output (the add_delta form)
+    y0 = torch.from_numpy(o.make_x(t, n, 5)).to(dev)
+    y1 = y0.clone()
+    ops.multi_delta_linear(p["x"], None, p["q"], p["s"], p["m"], p["ids"], bits=bits, out=y1, accumulate=True)
+    torch.cuda.synchronize()
+    ref_d = o.forward_ref(p["x_np"], None, p["dts"], p["ids_np"]) + y0.float().cpu().numpy()
+    assert o.rel_err(y1.cpu().numpy(), ref_d) <= TOL
+    # delta only, not accumulated: rows without a delta are zero
+    y2 = ops.multi_delta_linear(p["x"], None, p["q"], p["s"], p["m"], p["ids"], bits=bits)
+    torch.cuda.synchronize()
+    assert (y2[torch.from_numpy(p["ids_np"] < 0).to(dev)] == 0).all()
+    assert o.rel_err(y2.cpu().numpy(), o.forward_ref(p["x_np"], None, p["dts"], p["ids_np"])) <= TOL
+
+
+def test_build_tiles(dev):
+    from deltazip_amd import _lib
+    L = _lib.lib()
+    off = [0, 10, 10, 600, 601, 1113, 1113]          # S = 4: segments of 10, 0, 590, 1, 512, 0 rows
+    seg = torch.tensor(off, dtype=torch.int32, device=dev)
+    tiles = torch.full((12, 4), 77, dtype=torch.int32, device=dev)
+    assert L.dz_build_tiles(seg.data_ptr(), 5, tiles.data_ptr(), 12, torch.cuda.current_stream().cuda_stream) == 0
+    torch.cuda.synchronize()
+    got = tiles.cpu().tolist()
+    want = [[0, 10, -1, 0], [10, 266, 1, 0], [266, 522, 1, 0], [522, 600, 1, 0], [600, 601, 2, 0],
+            [601, 857, 3, 0], [857, 1113, 3, 0]]
+    assert got[:7] == want and all(r == [0, 0, -1, 0] for r in got[7:])
+    assert L.dz_build_tiles(None, 5, tiles.data_ptr(), 12, None) == -1
+    assert L.dz_build_tiles(seg.data_ptr(), 5000, tiles.data_ptr(), 12, None) == -2
