@@ -94,47 +94,70 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.w ? P.w : P.x), 0, 0x7fffffff, 0x00020000);
   const __amdgpu_buffer_rsrc_t rx =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.x), 0, 0x7fffffff, 0x00020000);
+  // base pass: slab s -> buffer s & 1, [weight slab | activation slab]
   auto issue = [&](int s, int buf) {
-    const bool base = s < nb;
-    const int soff = (base ? s : s - nb) * (BK * 2);
+    const int soff = s * (BK * 2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       unsigned char* dst = smem + buf * (2 * SLAB) + (wave * 4 + i) * 1024;
-      if (base)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
-                                                 (int)goff_w[i], soff, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
+                                               (int)goff_w[i], soff, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(dst + SLAB), 16,
+                                               (int)goff_x[i], soff, 0, 0);
+    }
+  };
+  // delta pass: activation slab sd -> stage sd & 3 of a ring of four (the same 128 KiB)
+  auto issue_xd = [&](int sd) {
+    const int soff = sd * (BK * 2);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      unsigned char* dst = smem + (sd & 3) * SLAB + (wave * 4 + i) * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)dst, 16,
                                                (int)goff_x[i], soff, 0, 0);
     }
   };
 
   // ---- packed delta operands: the 8 n-pairs (256 rows) of the workgroup's tile, one k-block at a
-  // time, staged in the weight half of an LDS buffer (idle during the delta pass): wavefront w
-  // fetches n-pair w -- 1 KiB of positions and 1 or 2 KiB of codes, already in lane order -- and
-  // every wavefront later reads the four n-pairs of its own feature half from there.
+  // time, staged in LDS behind the ring: wavefront w fetches n-pair w -- 1 KiB of positions and 1
+  // or 2 KiB of codes, already in lane order -- and every wavefront later reads the four n-pairs
+  // of its own feature half from there.
   constexpr int DT = (BITS == 2) ? 2048 : 3072;          // staged bytes per n-pair
+  unsigned char* const dstage = smem + 4 * SLAB;
+  const int slot_c = has_delta ? slot : 0;
+  const __amdgpu_buffer_rsrc_t rmeta = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u4_t*>(P.meta + (size_t)slot_c * P.meta_slot_u4), 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rcode = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<u4_t*>(P.codes + (size_t)slot_c * P.codes_slot_u4), 0, 0x7fffffff, 0x00020000);
+  const int np_w = min(n0 / DZ_NPAIR + wave, P.NP - 1);
   auto issue_delta = [&](int kb) {
-    unsigned char* dst = smem + (kb & 1) * (2 * SLAB) + wave * DT;
-    const int np = min(n0 / DZ_NPAIR + wave, P.NP - 1);
-    const size_t tile = (size_t)np * P.NKB + kb;
-    const char* mb = (const char*)(P.meta + (size_t)slot * P.meta_slot_u4 + tile * 64) + lane * 16;
-    const char* cb = (const char*)(P.codes + (size_t)slot * P.codes_slot_u4 + tile * (BITS == 2 ? 64 : 128)) + lane * 16;
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)mb,
-                                     (__attribute__((address_space(3))) void*)dst, 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)cb,
-                                     (__attribute__((address_space(3))) void*)(dst + 1024), 16, 0, 0);
+    unsigned char* dst = dstage + wave * DT;
+    const int tile = np_w * P.NKB + kb;
+    const int lo = lane * 16;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rmeta, (__attribute__((address_space(3))) void*)dst, 16, lo,
+                                             tile * 1024, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rcode, (__attribute__((address_space(3))) void*)(dst + 1024), 16, lo,
+                                             tile * (BITS == 2 ? 1024 : 2048), 0, 0);
     if (BITS == 4)
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(cb + 1024),
-                                       (__attribute__((address_space(3))) void*)(dst + 2048), 16, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rcode, (__attribute__((address_space(3))) void*)(dst + 2048), 16,
+                                               lo, tile * 2048 + 1024, 0, 0);
   };
-  // scales of scale group gi for the lane's 8 operand rows: row n0 + wn*128 + 16*t + i
-  // (two per register: entry p holds the scales of the two 16-row halves of n-pair p)
-  auto load_scales = [&](h2_t (&sc)[4], int gi) {
+  // scales of scale group gi: lane l fetches the scale of row 32*p + l % 32 of n-pair p (one
+  // 2-byte load per n-pair, nothing depends on it until the group starts); the two values a lane
+  // multiplies with -- rows i and 16 + i -- reach it by a cross-lane move when the group starts
+  auto load_scales = [&](int (&raw)[4], int gi) {
     const _Float16* sp = P.scales + (size_t)slot * P.scales_slot + (size_t)min(gi, P.G - 1) * P.N;
 #pragma unroll
+    for (int p = 0; p < 4; ++p)
+      raw[p] = *(const unsigned short*)(sp + min(n0 + wn * 128 + 32 * p + (lane & 31), P.N - 1));
+  };
+  auto spread_scales = [&](h2_t (&sc)[4], const int (&raw)[4]) {
+#pragma unroll
     for (int p = 0; p < 4; ++p) {
-      sc[p][0] = sp[min(n0 + wn * 128 + 32 * p + li, P.N - 1)];
-      sc[p][1] = sp[min(n0 + wn * 128 + 32 * p + 16 + li, P.N - 1)];
+      const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(li << 2, raw[p]) & 0xffffu;
+      const unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute((16 + li) << 2, raw[p]);
+      H2U u;
+      u.u = lo | (hi << 16);
+      sc[p] = u.h;
     }
   };
 
@@ -146,8 +169,17 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   for (int h = 0; h < 2; ++h) foff[h] = (((4 * h + lg) ^ ((li >> 1) & 7)) << 4);
   const int wrow = (wn * 128 + li) * 128, xrow = (wq * 64 + li) * 128;
 
-  if (total > 0) issue(0, 0);
-  if (nb == 0 && nd > 0) issue_delta(0);
+  // The delta pass starts with activation slabs 0 and 1 and the first k-block's packed operands
+  // already requested: at the start when there is no base pass, else during the last base slab
+  // (which sits in buffer 1 -- the slab count is a multiple of 4 -- so ring stages 0 and 1, the
+  // bytes of buffer 0, are free by then).
+  auto delta_prologue = [&]() {
+    issue_xd(0);
+    issue_xd(1);
+    issue_delta(0);
+  };
+  if (nb > 0) issue(0, 0);
+  else if (nd > 0) delta_prologue();
   // ---- base pass
   for (int s = 0; s < nb; ++s) {
     const int buf = s & 1;
@@ -155,10 +187,8 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     // the others (their shares are in, and nobody still reads the buffer filled next)
     __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0)
     __syncthreads();
-    if (s + 1 < total) issue(s + 1, buf ^ 1);
-    // the last base slab sits in buffer 1 (the slab count is a multiple of 4): the weight half of
-    // buffer 0 is free for the first k-block of the delta
-    if (s + 1 == nb && nd > 0) issue_delta(0);
+    if (s + 1 < nb) issue(s + 1, buf ^ 1);
+    else if (nd > 0) delta_prologue();
     if (!has_rows) continue;
     const unsigned char* wb = smem + buf * (2 * SLAB);
     const unsigned char* xb = wb + SLAB;
@@ -179,40 +209,49 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   }
   // ---- delta pass
   Frag<BITS> cur[4];
-  h2_t sc[4], scn[4];
+  h2_t sc[4];
+  int scn[4];
   if (nd > 0) load_scales(scn, 0);
   int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
   for (int sd = 0; sd < nd; ++sd) {
-    const int s = nb + sd, buf = s & 1;
     const int kb = sd >> 2, j = sd & 3;
-    __builtin_amdgcn_s_waitcnt(0x0070);
+    // Slab sd was requested three turns ago (slabs 0 and 1: before the pass).  Loads complete in
+    // order and at least the 8 requests of slabs sd + 1 and sd + 2 follow it, so "at most 8
+    // outstanding" means slab sd -- and anything requested before slab sd + 1, the staged k-block
+    // included -- has arrived.  s_waitcnt immediate: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8].
+    if (sd == 0 || sd + 1 >= nd) __builtin_amdgcn_s_waitcnt(0x0070);
+    else if (sd + 2 >= nd) __builtin_amdgcn_s_waitcnt(0x0074);
+    else __builtin_amdgcn_s_waitcnt(0x0078);
     __syncthreads();
-    if (s + 1 < total) issue(s + 1, buf ^ 1);
+    if (sd == 0) {
+      if (2 < nd) issue_xd(2);
+      if (3 < nd) issue_xd(3);
+    } else if (sd + 3 < nd) {
+      issue_xd(sd + 3);
+    }
     if (j == 0) {
-      // this k-block's packed operands were staged a k-block ago; the other staging area is free
-      // (every wavefront has passed the barrier above, so nobody reads it any more)
-      const unsigned char* dsrc = smem + (kb & 1) * (2 * SLAB) + (wn * 4) * DT + lane * 16;
+      // this k-block's packed operands were staged during the previous k-block
+      const unsigned char* dsrc = dstage + (wn * 4) * DT + lane * 16;
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
         cur[p].meta = *(const u4_t*)(dsrc + p * DT);
         cur[p].code[0] = *(const u4_t*)(dsrc + p * DT + 1024);
         if (BITS == 4) cur[p].code[BITS == 2 ? 0 : 1] = *(const u4_t*)(dsrc + p * DT + 2048);
       }
-      if (kb + 1 < P.NKB) issue_delta(kb + 1);
+    } else if (j == 1 && kb + 1 < P.NKB) {
+      // every wavefront has taken its copy (they all passed the barrier above): refill
+      issue_delta(kb + 1);
     }
     // scales: a scale group spans whole slabs (group size is a multiple of 64); the next group's
     // scales are requested during the last slab of the current one
-    if (gleft == P.gslabs) {
-#pragma unroll
-      for (int t = 0; t < 4; ++t) sc[t] = scn[t];
-    }
+    if (gleft == P.gslabs) spread_scales(sc, scn);
     if (gleft == 1 && sd + 1 < nd) load_scales(scn, gi + 1);
     if (--gleft == 0) {
       gleft = P.gslabs;
       ++gi;
     }
     if (!has_rows) continue;
-    const unsigned char* xb = smem + buf * (2 * SLAB) + SLAB;
+    const unsigned char* xb = smem + (sd & 3) * SLAB;
     h16_t B[4];
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
@@ -333,7 +372,7 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
-  const size_t lds = 2 * 2 * SLAB;
+  const size_t lds = 4 * SLAB + 8 * 3072;   // two base buffers = four ring stages, + staged k-block
   static bool attr_done[2] = {false, false};
   auto go = [&](auto kern, int which) -> int {
     if (!attr_done[which]) {
