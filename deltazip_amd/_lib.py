@@ -25,6 +25,7 @@ SIGNATURES = {
     "dz_embedding_select": (_i, [_vp, _vp, _vp, _vp, C.c_longlong, _i, _vp, _i, _i, _i, _i, _vp]),
     "dz_build_tiles": (_i, [_vp, _i, _vp, _i, _vp]),
     "dz_multi_delta_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "dz_compress_2of4": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dz_map_ids": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "dz_workspace_bytes": (_sz, [_i, _i, _i]),
     "dz_multi_delta_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,

@@ -257,3 +257,49 @@ def save_converted(tensors: Dict[str, torch.Tensor], compress_config: Compressio
     os.makedirs(save_dir, exist_ok=True)
     save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(save_dir, CHECKPOINT_NAME))
     compress_config.save_pretrained(save_dir)
+
+
+@torch.no_grad()
+def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: Dict[str, torch.Tensor],
+                   compress_config: CompressionConfig, device="cuda:0",
+                   pack_modules: Optional[Dict[str, Tuple[str, int]]] = None) -> Dict[str, torch.Tensor]:
+    """Fine-tuned model + base model -> serving-layout state dict of the compressed delta (what
+    `convert_model` makes of a checkpoint the reference's compressor wrote), on the GPU.
+
+    Every 2-D `*.weight` outside UNCOMPRESSED_MODULES is compressed as the reference's per-layer
+    step does it without calibration data: delta = target.float() - base.float()
+    (deltazip/core/sparsegpt.py:55-62), scales from the un-pruned delta, 2:4 pruning by magnitude,
+    round-to-nearest codes (`ops.compress_delta`).  The Hessian-weighted error feedback of
+    SparseGPT (sparsegpt.py:69-146), which needs calibration activations, is not applied.  The
+    remaining parameters are carried over from the fine-tuned model as they are, as the reference's
+    command line tool saves them (cli/compress.py:134-152)."""
+    if compress_config.bits not in (2, 4):
+        raise NotImplementedError("Only 2 and 4 bits are supported.")
+    if not (compress_config.prunen == 2 and compress_config.prunem == 4):
+        raise NotImplementedError("only 2:4 pruning (prunen=2, prunem=4) is supported")
+    pack_modules = PACK_MODULES if pack_modules is None else pack_modules
+    bits, gs = compress_config.bits, compress_config.group_size
+    out: Dict[str, torch.Tensor] = {}
+    native: Dict[str, Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]] = {}
+    for key, w in target_state_dict.items():
+        if key.endswith(".weight") and w.dim() == 2 and not any(u in key for u in UNCOMPRESSED_MODULES):
+            delta = w.to(device).float() - base_state_dict[key].to(device).float()
+            q, m, s = ops.compress_delta(delta.contiguous(), bits, gs)
+            native[key[: -len(".weight")]] = (q.cpu(), m.cpu(), s.cpu(), w.shape[1])
+        elif key.endswith(".weight") and any(u in key for u in UNCOMPRESSED_MODULES):
+            out[key[: -len(".weight")] + ".0.weight"] = w.detach().cpu()
+    plan: Dict[str, List[Tuple[int, str]]] = {}
+    for module, (q, m, s, K) in native.items():
+        hit = next((k for k in pack_modules if module.endswith("." + k) or module == k), None)
+        if hit is None:
+            out[module + ".0.qweight"], out[module + ".0.meta"], out[module + ".0.scales"] = q, m, s
+        else:
+            target, pos = pack_modules[hit]
+            plan.setdefault(module[: len(module) - len(hit)] + target, []).append((pos, module))
+    for target, members in plan.items():
+        members.sort()
+        if [p for p, _ in members] != list(range(len(members))):
+            raise ValueError(f"{target}: fused module has missing parts {[m for _, m in members]}")
+        q, m, s = _fuse_native([native[mod][:3] for _, mod in members], native[members[0][1]][3], bits, gs)
+        out[target + ".0.qweight"], out[target + ".0.meta"], out[target + ".0.scales"] = q, m, s
+    return out

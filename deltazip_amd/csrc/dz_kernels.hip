@@ -224,6 +224,120 @@ __global__ __launch_bounds__(256) void dz_embedding_select_kernel(const long lon
 }
 
 // ---------------------------------------------------------------------------------------------
+// compressor: fp32 delta [N, K] -> symmetric scales, 2:4 magnitude pruning, codes, native layout
+// ---------------------------------------------------------------------------------------------
+// One wavefront per (row, scale group): min / max of the group, then the symmetric parameters of
+// deltazip/core/quant.py:69-83 (perchannel, sym): the range is widened to [-m, m] when the group
+// has a negative value, an all-zero group gets [-1, 1], scale = (xmax - xmin) / maxq.
+__global__ __launch_bounds__(64) void dz_scales_kernel(const float* __restrict__ delta, int K, int N, int gs,
+                                                       int G, float maxq, float* __restrict__ scale32,
+                                                       _Float16* __restrict__ scale16) {
+  const int row = blockIdx.x / G, g = blockIdx.x % G, lane = threadIdx.x;
+  const float* p = delta + (size_t)row * K + (size_t)g * gs;
+  float mn = 0.f, mx = 0.f;
+  for (int c = lane * 4; c < gs; c += 256) {
+    const f4_t v = *(const f4_t*)(p + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mn = fminf(mn, v[e]);
+      mx = fmaxf(mx, v[e]);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o));
+    mx = fmaxf(mx, __shfl_xor(mx, o));
+  }
+  if (lane == 0) {
+    float xmin = mn, xmax = fmaxf(fabsf(mn), mx);
+    if (xmin < 0.f) xmin = -xmax;
+    if (xmin == 0.f && xmax == 0.f) {
+      xmin = -1.f;
+      xmax = 1.f;
+    }
+    const float sc = (xmax - xmin) / maxq;
+    scale32[(size_t)g * N + row] = sc;
+    scale16[(size_t)g * N + row] = (_Float16)sc;
+  }
+}
+
+// One wavefront per (n-pair, k-block) tile; lane 16*ga + i produces its own four words of the
+// native arrays from rows i and 16 + i, columns 64*j + 16*ga .. + 15 of the k-block.
+//   pruning   in every aligned group of 4 columns the 2 values of largest magnitude stay (ties:
+//             the lower column), the others become 0 -- deltazip/core/sparsegpt.py:123-135 with an
+//             identity Hessian
+//   codes     q = clamp(rint(x / scale) + zero, 0, maxq), fp32, zero = 2^(bits-1) -- quant.py:9-18
+//   positions the columns whose code differs from the zero-point, completed with the lowest
+//             remaining columns: what the repacker stores for the same codes
+template <int BITS>
+__global__ __launch_bounds__(64) void dz_compress_kernel(const float* __restrict__ delta,
+                                                         const float* __restrict__ scale32, int K, int N,
+                                                         int gs, uint32_t* __restrict__ codes,
+                                                         uint32_t* __restrict__ meta) {
+  const int nkb = K / DZ_KBLOCK;
+  const int np = blockIdx.x / nkb, kb = blockIdx.x % nkb;
+  const int la = threadIdx.x, ga = la >> 4, i = la & 15;
+  constexpr int zp = 1 << (BITS - 1);
+  constexpr float maxq = (float)((1 << BITS) - 1);
+  uint32_t mword[4] = {0u, 0u, 0u, 0u};
+  uint32_t cword[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col0 = kb * DZ_KBLOCK + 64 * j + 16 * ga;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      const int row = np * DZ_NPAIR + 16 * s + i;
+      const float sc = scale32[(size_t)(col0 / gs) * N + row];
+      const float* src = delta + (size_t)row * K + col0;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const f4_t v = *(const f4_t*)(src + 4 * p);
+        int c[4];
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+          int rank = 0;   // entries ahead of a: larger magnitude, or equal magnitude at a lower column
+#pragma unroll
+          for (int b = 0; b < 4; ++b)
+            if (b != a) rank += (b > a) ? (fabsf(v[b]) > fabsf(v[a])) : (fabsf(v[b]) >= fabsf(v[a]));
+          const float x = rank < 2 ? v[a] : 0.f;
+          const float qf = fminf(fmaxf(rintf(x / sc) + (float)zp, 0.f), maxq);
+          c[a] = (int)qf;
+        }
+        int pa = -1, pb = -1;
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          if (c[a] != zp) {
+            if (pa < 0) pa = a;
+            else if (pb < 0) pb = a;
+          }
+#pragma unroll
+        for (int a = 0; a < 4; ++a)
+          if (c[a] == zp) {
+            if (pa < 0) pa = a;
+            else if (pb < 0) pb = a;
+          }
+        const int lo = min(pa, pb), hi = max(pa, pb);
+        const uint32_t clo = (uint32_t)(lo == 0 ? c[0] : lo == 1 ? c[1] : c[2]);
+        const uint32_t chi = (uint32_t)(hi == 1 ? c[1] : hi == 2 ? c[2] : c[3]);
+        mword[j] |= ((uint32_t)lo << dz_meta_shift(s, 2 * p)) | ((uint32_t)hi << dz_meta_shift(s, 2 * p + 1));
+        if (BITS == 2) {
+          cword[0][j] |= (clo << dz_code2_shift(s, 2 * p)) | (chi << dz_code2_shift(s, 2 * p + 1));
+        } else {
+          cword[j >> 1][2 * (j & 1) + s] |= (clo << dz_code4_shift(2 * p)) | (chi << dz_code4_shift(2 * p + 1));
+        }
+      }
+    }
+  }
+  *(u4_t*)(meta + dz_meta_word(np, kb, la, 0, nkb)) = (u4_t){mword[0], mword[1], mword[2], mword[3]};
+  if (BITS == 2) {
+    *(u4_t*)(codes + dz_code2_word(np, kb, la, 0, nkb)) = (u4_t){cword[0][0], cword[0][1], cword[0][2], cword[0][3]};
+  } else {
+    *(u4_t*)(codes + dz_code4_word(np, kb, la, 0, 0, nkb)) = (u4_t){cword[0][0], cword[0][1], cword[0][2], cword[0][3]};
+    *(u4_t*)(codes + dz_code4_word(np, kb, la, 2, 0, nkb)) = (u4_t){cword[1][0], cword[1][1], cword[1][2], cword[1][3]};
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 int g_ksplit_override = 0;
@@ -344,6 +458,29 @@ int dz_embedding_select(const int64_t* tokens, const int64_t* indices, const uin
   hipLaunchKernelGGL(dz_embedding_select_kernel, dim3(T), dim3(256), 0, (hipStream_t)stream,
                      (const long long*)tokens, (const long long*)indices, (const _Float16*)base_weight,
                      (const _Float16*)weight_stack, stack_stride, S, V, H, (_Float16*)out, ldo);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size, void* out_codes,
+                     void* out_meta, uint16_t* out_scales, float* scale_workspace, void* stream) {
+  if (!delta || !out_codes || !out_meta || !out_scales || !scale_workspace) return DZ_EINVAL;
+  size_t cb, mb, sb;
+  int rc = dz_native_sizes(K, N, bits, group_size, &cb, &mb, &sb);
+  if (rc) return rc;
+  int gs;
+  if ((rc = check_group(K, group_size, &gs))) return rc;
+  if ((uintptr_t)delta & 15) return DZ_EALIGN;
+  const int G = K / gs;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(dz_scales_kernel, dim3((unsigned)N * G), dim3(64), 0, st, delta, K, N, gs, G,
+                     (float)((1 << bits) - 1), scale_workspace, (_Float16*)out_scales);
+  const unsigned tiles = (unsigned)(N / DZ_NPAIR) * (K / DZ_KBLOCK);
+  if (bits == 2)
+    hipLaunchKernelGGL(dz_compress_kernel<2>, dim3(tiles), dim3(64), 0, st, delta, scale_workspace, K, N, gs,
+                       (uint32_t*)out_codes, (uint32_t*)out_meta);
+  else
+    hipLaunchKernelGGL(dz_compress_kernel<4>, dim3(tiles), dim3(64), 0, st, delta, scale_workspace, K, N, gs,
+                       (uint32_t*)out_codes, (uint32_t*)out_meta);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 

@@ -192,6 +192,29 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     return out
 
 
+def compress_delta(delta: torch.Tensor, bits: int, group_size: int = -1):
+    """fp32 delta [N, K] on the GPU -> (qweight, meta, scales) of one slot in the native layout:
+    symmetric scales from the un-pruned values, 2:4 magnitude pruning, round-to-nearest codes
+    (deltazip/core/quant.py:9-18, 48-130; core/sparsegpt.py:64-66, 123-135 with an identity
+    Hessian).  The same bytes as compressing and packing the reference's way and converting with
+    `repack_gptq_to_native`."""
+    _need_cuda(delta)
+    if bits not in (2, 4):
+        raise NotImplementedError("Only 2 and 4 bits are supported.")
+    if delta.dtype != torch.float32 or delta.dim() != 2 or not delta.is_contiguous():
+        raise ValueError("delta must be a contiguous float32 [N, K] tensor")
+    N, K = delta.shape
+    qs, ms, ss = stacked_shapes(K, N, bits, group_size)
+    q = torch.empty(qs, dtype=torch.int32, device=delta.device)
+    m = torch.empty(ms, dtype=torch.int16, device=delta.device)
+    s = torch.empty(ss, dtype=torch.float16, device=delta.device)
+    ws = torch.empty(ss, dtype=torch.float32, device=delta.device)
+    rc = _lib.lib().dz_compress_2of4(delta.data_ptr(), K, N, bits, group_size, q.data_ptr(), m.data_ptr(),
+                                     s.data_ptr(), ws.data_ptr(), _stream())
+    _lib.check(rc, "dz_compress_2of4")
+    return q, m, s
+
+
 def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_ids: torch.Tensor,
             max_deltas: int, vocab_size: int, extra_vocab_size: int, base_indices: torch.Tensor,
             sampler_indices: Optional[torch.Tensor] = None,

@@ -109,6 +109,18 @@ int dz_embedding_select(const int64_t* tokens, const int64_t* indices, const uin
                         const uint16_t* weight_stack, long long stack_stride, int S, uint16_t* out, int T,
                         int V, int H, int ldo, void* stream);
 
+/* Compress one delta on the device: delta [N, K] fp32 row-major -> native codes / positions /
+ * fp16 scales.  Symmetric scales per output row (group_size -1) or per (row, group) from the
+ * un-pruned values (deltazip/core/quant.py:48-130 sym branch; sparsegpt.py:64-66), 2:4 pruning
+ * by magnitude (sparsegpt.py:123-135 with an identity Hessian; ties keep the lower column), codes
+ * q = clamp(rint(x / scale) + 2^(bits-1), 0, 2^bits - 1) with the fp32 scale (quant.py:9-18),
+ * stored scale = fp16(scale) (qlinear_cuda.py:153-156).  The result equals, byte for byte, what
+ * dz_repack_2of4 makes of the same delta compressed and packed the reference's way.  The
+ * Hessian-weighted solve of SparseGPT (sparsegpt.py:69-146) is not part of this.
+ * scale_workspace: G * N floats of device memory (G = K / group_size, 1 for -1). */
+int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size, void* out_codes,
+                     void* out_meta, uint16_t* out_scales, float* scale_workspace, void* stream);
+
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
  * zero-filled once before first use; calls leave it ready for the next call.  Calls that share
  * a workspace must be ordered on one stream. */

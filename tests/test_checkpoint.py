@@ -141,3 +141,44 @@ def test_unsupported_checkpoints_are_refused(dzlib):
            for key, v in (("qweight", qw), ("qzeros", qz), ("scales", sc), ("g_idx", gi))}
     with pytest.raises(ValueError):
         ck.convert_model(bad, bits=4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,gs", [(4, -1), (2, 128)])
+def test_compress_model_on_gpu(dev, bits, gs):
+    """Base + fine-tuned state dicts -> compressed serving-layout delta on the GPU; every fused
+    module dequantises to what the reference's pipeline (restated by the oracle) gives for its
+    parts, and the result loads like a checkpoint."""
+    g = torch.Generator().manual_seed(11)
+    base, target = {}, {}
+    for name, (n, k) in SHAPES.items():
+        key = f"model.layers.0.{name}.weight"
+        base[key] = (torch.randn(n, k, generator=g) * 0.02).half()
+        target[key] = (base[key].float() + torch.randn(n, k, generator=g) * 1e-3).half()
+    for key, shape in (("model.embed_tokens.weight", (V, H)), ("lm_head.weight", (V, H)), ("model.norm.weight", (H,)),
+                       ("model.layers.0.input_layernorm.weight", (H,))):
+        base[key] = torch.randn(*shape, generator=g).half()
+        target[key] = torch.randn(*shape, generator=g).half()
+    cfg = ck.CompressionConfig(bits=bits, group_size=gs, sparsity=0.5, prunen=2, prunem=4)
+    out = ck.compress_model(base, target, cfg, device=dev)
+    want = {}
+    for name, (n, k) in SHAPES.items():
+        key = f"model.layers.0.{name}.weight"
+        d32 = target[key].float().numpy() - base[key].float().numpy()
+        codes, scales16, zeros, _ = o.compress_delta(d32, bits, gs)
+        qw, qz, sc, gi = o.pack_codes_gptq(codes, zeros, scales16, bits)
+        want[name] = o.dequant_gptq(qw, qz, sc, gi, bits).T
+    fused = {"self_attn.qkv_proj": ["self_attn.q_proj", "self_attn.k_proj", "self_attn.v_proj"],
+             "mlp.gate_up_proj": ["mlp.gate_proj", "mlp.up_proj"],
+             "self_attn.o_proj": ["self_attn.o_proj"], "mlp.down_proj": ["mlp.down_proj"]}
+    for tname, parts in fused.items():
+        ref = np.concatenate([want[x] for x in parts], axis=0)
+        q, m, s = (out[f"model.layers.0.{tname}.0.{x}"] for x in ("qweight", "meta", "scales"))
+        got = native_dequant(q, m, s, ref.shape[1], bits)
+        assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(ref).view(np.uint16)), tname
+    assert torch.equal(out["model.embed_tokens.0.weight"], target["model.embed_tokens.weight"])
+    assert torch.equal(out["model.layers.0.input_layernorm.0.weight"], target["model.layers.0.input_layernorm.weight"])
+    dm = ck.DeltaModel.from_tensors(out, 3, cfg, pin_memory=False)
+    assert dm.get_delta("model.layers.0.self_attn.qkv_proj")._compressed and not dm.get_delta("lm_head")._compressed
+    with pytest.raises(NotImplementedError):
+        ck.compress_model(base, target, ck.CompressionConfig(bits=4, prunen=0, prunem=0), device=dev)

@@ -335,3 +335,41 @@ def test_build_tiles(dev):
     assert got[:7] == want and all(r == [0, 0, -1, 0] for r in got[7:])
     assert L.dz_build_tiles(None, 5, tiles.data_ptr(), 12, None) == -1
     assert L.dz_build_tiles(seg.data_ptr(), 5000, tiles.data_ptr(), 12, None) == -2
+
+
+@pytest.mark.parametrize("n,k,bits,gs", [(32, 256, 4, -1), (64, 512, 2, -1), (96, 768, 4, 128), (160, 1024, 2, 64),
+                                         (256, 2048, 4, 256)])
+def test_compressor_matches_reference_pipeline(dev, n, k, bits, gs):
+    """dz_compress_2of4 against the oracle's restatement of the reference's pipeline (scales from the
+    un-pruned delta, 2:4 by magnitude, quantise, GPTQ pack) followed by the repacker: same bytes.
+    Rows that are all zero, rows without a negative value, magnitude ties and values that quantise to
+    the zero-point are all present."""
+    rng = np.random.default_rng(n + k + bits)
+    d = (rng.standard_normal((n, k)) * 1e-3).astype(np.float32)
+    d[3] = 0.0                                        # all-zero row: range (-1, 1)
+    d[5] = np.abs(d[5])                               # no negative value: range (0, max)
+    d[7, :64] = np.float32(2e-3) * rng.integers(-2, 3, 64)   # many exact ties and exact zeros
+    d[9] *= 1e-4                                      # tiny values next to ...
+    d[9, 17] = 1.0                                    # ... one large one: most codes are the zero-point
+    codes, scales16, zeros, keep = o.compress_delta(d, bits, gs)
+    qw, qz, sc, gi = o.pack_codes_gptq(codes, zeros, scales16, bits)
+    want_c, want_m, want_s = o.repack_native(qw, qz, sc, gi, bits)
+    q, m, s = ops.compress_delta(torch.from_numpy(d).to(dev), bits, gs)
+    torch.cuda.synchronize()
+    assert q.cpu().numpy().view(np.uint32).tobytes() == want_c.tobytes()
+    assert m.cpu().numpy().view(np.uint32).tobytes() == want_m.tobytes()
+    assert np.array_equal(s.cpu().numpy().view(np.uint16), want_s.view(np.uint16))
+    # and it dequantises (on the GPU) to the reference dequantisation of those GPTQ tensors
+    got = ops.dequant(q, m, s, k, n, bits).cpu().numpy()
+    assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(o.dequant_gptq(qw, qz, sc, gi, bits).T).view(np.uint16))
+
+
+def test_compressor_argument_checks(dev):
+    with pytest.raises(ValueError):
+        ops.compress_delta(torch.zeros(32, 256, device=dev, dtype=torch.float16), 4)
+    with pytest.raises(NotImplementedError):
+        ops.compress_delta(torch.zeros(32, 256, device=dev), 3)
+    with pytest.raises(ValueError):
+        ops.compress_delta(torch.zeros(32, 200, device=dev), 4)
+    with pytest.raises(ValueError):
+        ops.compress_delta(torch.zeros(32, 256), 4)
