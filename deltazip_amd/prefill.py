@@ -46,6 +46,15 @@ def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked,
     S = qweight_stacked.shape[0]
     G = scales_stacked[0].numel() // N
     group_size = -1 if G == 1 else K // G
+    # the kernel addresses an operand with 31-bit byte offsets: very long batches go in pieces
+    max_rows = ((1 << 31) - 1) // (2 * K)
+    if T > max_rows:
+        step = max(256, max_rows // 256 * 256)
+        for r in range(0, T, step):
+            multi_delta_linear_prefill(x2[r:r + step], base_weight, qweight_stacked, scales_stacked, meta_stacked,
+                                       indices[r:r + step].contiguous(), bits=bits, out=out[r:r + step],
+                                       accumulate=accumulate)
+        return out
     lib = _lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
     perm, seg_off = segment(indices, S)
