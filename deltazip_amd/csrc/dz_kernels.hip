@@ -338,6 +338,87 @@ __global__ __launch_bounds__(64) void dz_compress_kernel(const float* __restrict
 }
 
 // ---------------------------------------------------------------------------------------------
+// 33..128 tokens: the order in which the fused kernel takes the tokens, 32 per chunk.  Tokens of
+// one delta stay together, and the chunks are made to meet about the same number of distinct
+// deltas (the kernel's time per chunk grows with that number; a plain cut of the id-sorted order
+// puts one popular delta alone into a chunk and all the rare ones together into another).
+// The segments -- one per delta present -- are ranked by size; counting from the largest, segment
+// r goes to group r mod nchunk; the groups are laid out one after the other, each smallest
+// segment first, and the chunks are the 32-token cuts of that layout.  Every group holds the same
+// number of segments and group g is at least as long as group g + 1, so a cut falls into the tail
+// of a group: what spills into the next chunk is part of a popular delta, not several rare ones.
+// One workgroup, one thread per token, everything by counting over the (at most 128) tokens: no
+// per-slot table, so any number of slots is fine.
+// ---------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(128) void dz_deal_kernel(const long long* __restrict__ idx, int T, int S,
+                                                      int* __restrict__ perm_out) {
+  __shared__ __attribute__((aligned(16))) int s_key[128], s_size[128], s_dkey[128];
+  __shared__ int s_pos[128], s_wcount[2];
+  const int tid = threadIdx.x;
+  const int nchunk = (T + 31) / 32;
+  int key = 0x7fffffff;   // threads beyond T hold no token; their entries never match or count
+  if (tid < T) {
+    const long long id = idx[tid];
+    key = (id < 0 || id >= S) ? 0 : (int)id + 1;
+  }
+  s_key[tid] = key;
+  __syncthreads();
+  // Tables are read four entries per LDS read with several reads in flight (a loop that takes one
+  // entry per turn waits out the LDS latency every time).
+  typedef int i4_t __attribute__((ext_vector_type(4)));
+  // my segment: its size, my place in it, its first token (the segment's "leader")
+  int size = 0, rin = 0, leader = tid;
+#pragma unroll 8
+  for (int q = 0; q < 32; ++q) {
+    const i4_t v = ((const i4_t*)s_key)[q];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int j = 4 * q + e;
+      const bool same = v[e] == key;
+      size += same;
+      rin += same && j < tid;
+      leader = (same && j < leader) ? j : leader;
+    }
+  }
+  const bool is_leader = tid < T && leader == tid;
+  // the segments, compacted (order of their first tokens): size | first token << 8; zero-padded
+  const unsigned long long lm = __builtin_amdgcn_ballot_w64(is_leader);
+  const int lane = tid & 63, wave = tid >> 6;
+  if (lane == 0) s_wcount[wave] = __builtin_popcountll(lm);
+  s_size[tid] = 0;
+  s_dkey[tid] = 0x7fffffff;
+  __syncthreads();
+  const int nseg = s_wcount[0] + s_wcount[1];
+  const int slot = (wave ? s_wcount[0] : 0) + __builtin_popcountll(lm & ((1ull << lane) - 1ull));
+  if (is_leader) s_size[slot] = size | (tid << 8);
+  __syncthreads();
+  const int nq = (nseg + 3) >> 2;
+  // leaders: rank of the segment by (size, first token)
+  int rank = 0;
+  for (int q = 0; q < nq; ++q) {
+    const i4_t v = ((const i4_t*)s_size)[q];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int sj = v[e] & 0xff, fj = v[e] >> 8;
+      rank += v[e] != 0 && (sj < size || (sj == size && fj < tid));
+    }
+  }
+  const int dkey = is_leader ? ((((nseg - 1 - rank) % nchunk) << 16) | rank) : 0x7fffffff;
+  if (is_leader) s_dkey[slot] = dkey;
+  __syncthreads();
+  int pos = 0;   // tokens of the segments laid out before mine
+  for (int q = 0; q < nq; ++q) {
+    const i4_t d = ((const i4_t*)s_dkey)[q];
+    const i4_t z = ((const i4_t*)s_size)[q];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) pos += (d[e] < dkey) ? (z[e] & 0xff) : 0;
+  }
+  s_pos[tid] = pos;
+  __syncthreads();
+  if (tid < T) perm_out[s_pos[leader] + rin] = tid;
+}
+
+// ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
 int g_ksplit_override = 0;
@@ -352,7 +433,7 @@ inline int check_group(int K, int group_size, int* gs_out) {
 constexpr size_t WS_HEADER = 256;  // status word
 inline size_t ws_counter_bytes(int N) { return (((size_t)(N / DZ_NPAIR + 8) * 4 * 4) + 255) / 256 * 256; }   // 4 chunks
 constexpr int MAX_KSPLIT = 16;
-constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // segment offsets + token order
+constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // reserved + token order
 
 }  // namespace
 
@@ -533,10 +614,9 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
   P.perm = nullptr;
   P.tok0 = 0;
   if (T <= 32) return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
-  // 33..128 tokens: order the tokens by delta id on the device (no host round trip), so that each
-  // chunk of 32 meets as few deltas as possible; one launch carries all chunks
-  if (S > DZ_MAX_SLOTS_SEGMENT) return DZ_ESHAPE;
-  if ((rc = dz_segment(indices, T, S, perm, seg_off, stream))) return rc;
+  // 33..128 tokens: group the tokens by delta id on the device (no host round trip) and deal the
+  // groups to the chunks of 32; one launch carries all chunks
+  hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
   P.perm = perm;
   return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
 }

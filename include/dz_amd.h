@@ -131,9 +131,10 @@ size_t dz_workspace_bytes(int T, int K, int N);
  * indices [T] int64, -1 = base only, read on the device at execution time; y [T, ldy] fp16,
  * columns 0..N-1 written.  accumulate = 0: y = result; 1: y += result (fp32 add, one rounding).
  * Stands in for sbmm_4bit_2_4_native / ibmm_sparse_marlin at the call sites listed above.
- * Requires 1 <= T <= DZ_MAX_TOKENS_FUSED and, above 32 tokens, S <= DZ_MAX_SLOTS_SEGMENT (the
- * tokens are then ordered by id on the device and handled 32 at a time, in one launch).  Larger
- * batches are served by the host wrapper from dz_segment + dz_dequant + dz_gemm_f16_grouped. */
+ * Requires 1 <= T <= DZ_MAX_TOKENS_FUSED; above 32 tokens the tokens are grouped by id on the
+ * device and handled 32 at a time, in one launch, the groups dealt so that every 32 meet about
+ * the same number of deltas.  Larger batches are served by the host wrapper from dz_segment +
+ * dz_build_tiles + dz_multi_delta_gemm. */
 int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
                           const void* codes_stacked, const void* meta_stacked,
                           const void* scales_stacked, const int64_t* indices, uint16_t* y,

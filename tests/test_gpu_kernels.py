@@ -285,6 +285,34 @@ def test_unsorted_batches_above_32_tokens(dev, t):
     assert ops.workspace_status() == 0
 
 
+@pytest.mark.parametrize("t,kind", [(64, "zipf"), (128, "zipf"), (100, "single"), (77, "uniform")])
+def test_dealt_chunks_skewed_mixes_and_many_slots(dev, t, kind):
+    """33..128 tokens: the tokens are dealt to the 32-token chunks by delta (popular deltas split,
+    rare ones spread); whatever the mix, every token must get its own delta's result in its own
+    row -- also with far more slots than the sort used for long batches can take, most of them
+    empty."""
+    nd = 24
+    p = make_problem(64, 512, 2, -1, nd, t, kind, 5150 + t, dev)
+    S = 1000                                         # slots; deltas sit in scattered ones
+    where = np.random.default_rng(t).choice(S, nd, replace=False)
+    q = torch.zeros((S,) + tuple(p["q"].shape[1:]), dtype=p["q"].dtype, device=dev)
+    m = torch.zeros((S,) + tuple(p["m"].shape[1:]), dtype=p["m"].dtype, device=dev)
+    s = torch.zeros((S,) + tuple(p["s"].shape[1:]), dtype=p["s"].dtype, device=dev)
+    idx = torch.from_numpy(where).to(dev)
+    q[idx], m[idx], s[idx] = p["q"], p["m"], p["s"]
+    ids_np = p["ids_np"].copy()
+    slots_np = np.where(ids_np >= 0, where[np.maximum(ids_np, 0)], -1)
+    slots_np[5] = -1
+    ids_np[5] = -1
+    perm = np.random.default_rng(t + 1).permutation(t)          # arbitrary arrival order
+    y = ops.apply_delta(p["x"][torch.from_numpy(perm).to(dev)], q, s, m, torch.from_numpy(slots_np[perm]).to(dev),
+                        p["wb"])
+    torch.cuda.synchronize()
+    ref = o.forward_ref(p["x_np"][perm], p["wb_np"], p["dts"], ids_np[perm])
+    assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+    assert ops.workspace_status() == 0
+
+
 PREFILL_CASES = [
     # n, k, bits, gs, deltas, tokens, ids
     (256, 1024, 2, -1, 4, 400, "uniform"),
