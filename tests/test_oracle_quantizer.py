@@ -88,3 +88,22 @@ def test_compressed_delta_is_2of4(bits):
     assert np.all((c == zp).sum(axis=2) >= 2)          # at least two zero-point codes per group
     assert np.all(keep.reshape(32, 64, 4).sum(axis=2) == 2)
     assert np.all(codes.T[~keep] == zp)                # pruned entries carry the zero-point
+
+
+def test_compress_delta_known_answers():
+    """The chain scales-from-unpruned -> 2:4 by magnitude -> quantise, on a row worked out by hand:
+    b = 4: scale = 2 * 0.003 / 15 = 4e-4; 0.003 and -0.0029 stay; 0.003 / 4e-4 = 7.5 -> 8 (half to
+    even) + 8 = 16 -> 15; -0.0029 / 4e-4 = -7.25 -> -7 + 8 = 1; the pruned pair carries the zero-point.
+    b = 2: scale = 2e-3; 1.5 -> 2 + 2 = 4 -> 3; -1.45 -> -1 + 2 = 1."""
+    row = np.array([[0.003, -0.001, 0.0005, -0.0029]], dtype=np.float32)
+    codes, scales16, zeros, keep = o.compress_delta(row, 4)
+    assert codes.T.tolist() == [[15, 8, 8, 1]] and keep.tolist() == [[True, False, False, True]]
+    assert zeros.tolist() == [[8]] and scales16.view(np.uint16)[0, 0] == np.float16(4e-4).view(np.uint16)
+    codes, scales16, zeros, keep = o.compress_delta(row, 2)
+    assert codes.T.tolist() == [[3, 2, 2, 1]] and zeros.tolist() == [[2]]
+    # the scale comes from the un-pruned row: a large value that is pruned away still sets it
+    row = np.array([[0.004, 0.004, 0.004, -0.004, 0.0, 0.0, 0.001, 0.0]], dtype=np.float32)
+    codes, scales16, _, keep = o.compress_delta(row, 4)
+    assert keep.tolist() == [[True, True, False, False, True, False, True, False]]
+    # scale = 0.008 / 15; 0.004 / scale = 7.5 -> 8 -> 16 -> 15; 0.001 / scale = 1.875 -> 2 -> 10
+    assert codes.T.tolist() == [[15, 15, 8, 8, 8, 8, 10, 8]]
