@@ -33,10 +33,10 @@ SHAPES = [("q_proj", 4096, 4096), ("k_proj", 4096, 4096), ("v_proj", 4096, 4096)
 T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1    # the default workload (configuration 2)
 
 
-# HBM bytes per launch (average over the 7 launches of a step) of the default workload, from
+# HBM bytes per launch (average over the 4 launches of a step) of the default workload, from
 # rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what the same counter
 # reads for the --calib-copy-mib copy kernel; the figures are in profiles/*__hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 124070000
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 216875455
 
 
 def algorithmic_bytes(K, N, T, bits, d_present, G=1):
@@ -110,7 +110,8 @@ CONFIGS = {
     1: dict(name="4096->4096, 1 token, one 4-bit delta (per-channel scales)", shapes=[("linear", 4096, 4096)],
             T=1, S=1, bits=4, gs=-1, ids="zeros", bound="hbm"),
     2: dict(name="Llama-2-7B decode projections (q,k,v,o 4096->4096; gate,up 4096->11008; down 11008->4096), "
-                 "one step = these 7 multi-delta linear calls; 32 tokens, 8 deltas (2-bit, 2:4 sparse, "
+                 "one step = these 7 multi-delta linears (q/k/v in one launch, gate/up in one launch, as the "
+                 "reference's fused layers run them; --separate-launches: 7 launches); 32 tokens, 8 deltas (2-bit, 2:4 sparse, "
                  "per-channel fp16 scales), ids uniform over the deltas",
             shapes=SHAPES, T=32, S=8, bits=2, gs=-1, ids="uniform", bound="hbm"),
     3: dict(name="Llama-2-7B projections, 64 tokens, 32 deltas (4-bit, 2:4, group size 128), Zipf(1.5) ids",
@@ -146,6 +147,9 @@ def main():
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ksplit", type=int, default=0)
+    ap.add_argument("--separate-launches", action="store_true",
+                    help="one launch per projection (default: q/k/v and gate/up, which share their input in a "
+                         "decoder layer and which the reference holds as fused layers, go in one launch each)")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="before the timed region, run a plain elementwise copy kernel over this many MiB "
                          "(reads and writes that much): the yardstick for scaling FETCH_SIZE / WRITE_SIZE counters")
@@ -187,34 +191,66 @@ def main():
     ops.set_ksplit(args.ksplit)
     fused = T <= 128
 
+    # launches of a step: q/k/v in one, o, gate/up in one, down (the reference runs q/k/v and gate/up as
+    # fused layers: serving/vllm/delta/layers_marlin.py:281-487); --separate-launches: one per projection
+    names = [sh[0] for sh in shapes]
+    groups = [[j] for j in range(len(shapes))]
+    if fused and not args.separate_launches and names == [sh[0] for sh in SHAPES]:
+        groups = [[0, 1, 2], [3], [4, 5], [6]]
+
     if fused:
         # pre-marshalled C-ABI calls (device pointers and sizes only)
-        ws_bytes = max(lib.dz_workspace_bytes(T, K, N) for _, K, N in shapes)
+        ws_bytes = max(lib.dz_workspace_bytes(T, shapes[g[0]][1], sum(shapes[j][2] for j in g)) for g in groups)
         ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-        f = lib.dz_multi_delta_linear
+        f, fb = lib.dz_multi_delta_linear, lib.dz_multi_delta_linear_batch
         vp = C.c_void_p
+        keep = []                                   # the pointer arrays must outlive the calls
         prepared = []
+        single = []                                 # every projection as a launch of its own (per-shape timing)
         for calls in layers:
             pc = []
-            for name, K, N, x, wb, q, m, s, y in calls:
-                pc.append((vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
-                           vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
-                           vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream)))
+            for g in groups:
+                if len(g) == 1:
+                    name, K, N, x, wb, q, m, s, y = calls[g[0]]
+                    pc.append((f, (vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()),
+                                   vp(s.data_ptr()), vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
+                                   vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))))
+                else:
+                    n = len(g)
+                    arr = lambda k: (vp * n)(*[calls[j][k].data_ptr() for j in g])
+                    ax, aw, aq, am, asc, ay = arr(3), arr(4), arr(5), arr(6), arr(7), arr(8)
+                    an = (C.c_int * n)(*[calls[j][2] for j in g])
+                    keep.append((ax, aw, aq, am, asc, ay, an))
+                    pc.append((fb, (n, ax, aw, aq, am, asc, vp(ids.data_ptr()), ay, an, an, T, calls[g[0]][1], S, bits,
+                                    gs, 0, vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))))
             prepared.append(pc)
+            single.append([(vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
+                            vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
+                            vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))
+                           for name, K, N, x, wb, q, m, s, y in calls])
+
+        def launch(i, gi):
+            fn, a = prepared[i % len(prepared)][gi]
+            rc = fn(*a)
+            if rc:
+                raise RuntimeError(f"multi-delta linear launch failed: {lib.dz_strerror(rc).decode()}")
 
         def call(i, idx):
-            rc = f(*prepared[i % len(prepared)][idx])
+            rc = f(*single[i % len(single)][idx])
             if rc:
                 raise RuntimeError(f"dz_multi_delta_linear failed: {lib.dz_strerror(rc).decode()}")
     else:
-        # prefill-sized: the host wrapper segments the batch and runs dequant + pair-GEMM per delta
+        # prefill-sized: the host wrapper groups the batch and runs the packed-delta GEMM
         def call(i, idx):
             name, K, N, x, wb, q, m, s, y = layers[i % len(layers)][idx]
             ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y)
 
+        def launch(i, gi):
+            call(i, groups[gi][0])
+
     def step(i):
-        for idx in range(len(shapes)):
-            call(i, idx)
+        for gi in range(len(groups)):
+            launch(i, gi)
 
     if args.calib_copy_mib > 0:
         src = torch.ones(args.calib_copy_mib << 19, dtype=torch.float16, device=dev)
@@ -239,8 +275,8 @@ def main():
 
     def abytes(K, N):
         return algorithmic_bytes(K, N, T, bits, d_present, 1 if gs == -1 else K // gs)
-    default_workload = args.config == 2 and not args.unsorted and args.ksplit == 0
-    launches = steps * len(shapes)
+    default_workload = args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
+    launches = steps * len(groups)
     step_bytes = sum(abytes(K, N) for _, K, N in shapes)
     step_flops = sum(2.0 * T * K * N for _, K, N in shapes)
     avg_launch_s = gpu_s / launches              # includes the gaps between consecutive launches
@@ -264,20 +300,20 @@ def main():
         per_call_us[f"{K}x{N}"] = ent
 
     if cfg["bound"] == "hbm":
-        achieved = (step_bytes / len(shapes)) / avg_launch_s / 1e9
+        achieved = (step_bytes / len(groups)) / avg_launch_s / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
-                    "kernel": "dz_mdl32_kernel",
-                    "algorithmic_bytes_per_launch": step_bytes // len(shapes),
+                    "kernel": "dz_mdl32_kernel" if all(len(g) == 1 for g in groups) else "dz_mdl32_kernel + dz_mdl32_batch_kernel (same body)",
+                    "algorithmic_bytes_per_launch": step_bytes // len(groups),
                     "avg_launch_us": round(avg_launch_s * 1e6, 2)}
     else:
         # base contraction only (2*T*K*N per call); the per-delta dequantisation and the delta half of
         # the pair-GEMM are extra work inside the same time
-        achieved = (step_flops / len(shapes)) / avg_launch_s / 1e12
+        achieved = (step_flops / len(groups)) / avg_launch_s / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
                     "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
-                    "kernel": "dz_gemm24_kernel", "algorithmic_flops_per_call": step_flops / len(shapes),
+                    "kernel": "dz_gemm24_kernel", "algorithmic_flops_per_call": step_flops / len(groups),
                     "avg_call_us": round(avg_launch_s * 1e6, 2)}
 
     out = {
@@ -291,8 +327,9 @@ def main():
         "config": {"workload": cfg["name"] + ("" if args.unsorted or cfg["ids"] in ("zeros", "blocks")
                                               else ", batch sorted by delta id"),
                    "baseline_config": args.config, "tokens": T, "deltas": S, "deltas_present": d_present,
-                   "bits": bits, "group_size": gs, "layers_resident": nlayers, "launches_per_step": len(shapes)},
-        "us_per_layer_call": round(avg_launch_s * 1e6, 2),
+                   "bits": bits, "group_size": gs, "layers_resident": nlayers, "launches_per_step": len(groups),
+                   "launches": ["+".join(names[j] for j in g) for g in groups]},
+        "us_per_layer_call": round(gpu_s / (steps * len(shapes)) * 1e6, 2),
         "per_shape": per_call_us,
         "roofline": roofline,
         "parity": parity,

@@ -94,6 +94,14 @@ struct MdlParams {
   int NP, NKB, NPG;
 };
 
+// Up to DZ_MAX_BATCH layer calls in one launch; np_end[j] = n-pairs of calls 0..j (entries beyond
+// the last call repeat the total).
+constexpr int DZ_MAX_BATCH = DZ_MAX_BATCH_CALLS;
+struct MdlBatch {
+  MdlParams p[DZ_MAX_BATCH];
+  int np_end[DZ_MAX_BATCH];
+};
+
 constexpr int XS = DZ_KBLOCK + 8;  // LDS row stride of the staged activations, in halves
 
 template <int BITS>
@@ -124,3 +132,4 @@ __device__ __forceinline__ Frag<BITS> load_frag(const MdlParams& P, int d, int n
 
 // Launch of the T <= 32 kernel (dz_mdl32.hip).
 int dz_launch_mdl32(const MdlParams& P, int bits, bool pre, hipStream_t st, int ksplit_override);
+int dz_launch_mdl32_batch(const MdlParams* P, int nprob, int bits, bool pre, hipStream_t st, int ksplit_override);

@@ -565,11 +565,75 @@ int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size,
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
-// workspace: [status 256 B][segment offsets + token order][arrival counters][partial sums]
+// workspace: [status 256 B][token order][per call: arrival counters | partial sums]
+constexpr size_t WS_BATCH_SLACK = 4096;   // rounding of the per-call regions of a batch
 size_t dz_workspace_bytes(int T, int K, int N) {
   (void)K;
   if (T < 1 || N < 1) return 0;
-  return WS_HEADER + WS_PERM_BYTES + ws_counter_bytes(N) + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
+  return WS_HEADER + WS_PERM_BYTES + ws_counter_bytes(N) + WS_BATCH_SLACK + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
+}
+
+int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
+                                const void* const* codes_stacked, const void* const* meta_stacked,
+                                const void* const* scales_stacked, const int64_t* indices,
+                                uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
+                                int bits, int group_size, int accumulate, void* workspace,
+                                size_t workspace_bytes, void* stream) {
+  if (ncalls < 1 || ncalls > DZ_MAX_BATCH_CALLS) return DZ_ESHAPE;
+  if (!x || !w_base || !codes_stacked || !meta_stacked || !scales_stacked || !indices || !y || !N || !ldy)
+    return DZ_EINVAL;
+  if (S < 1) return DZ_EINVAL;  // at least one slot: the kernels always address slot 0
+  if (T < 1 || T > DZ_MAX_TOKENS_FUSED) return DZ_ESHAPE;
+  int gs, rc;
+  if ((rc = check_group(K, group_size, &gs))) return rc;
+  long long n_total = 0;
+  for (int j = 0; j < ncalls; ++j) {
+    size_t cb, mb, sb;
+    if ((rc = dz_native_sizes(K, N[j], bits, group_size, &cb, &mb, &sb))) return rc;
+    if (!x[j] || !y[j] || !codes_stacked[j] || !meta_stacked[j] || !scales_stacked[j]) return DZ_EINVAL;
+    if (ldy[j] < N[j] || ldy[j] % 4) return DZ_ESHAPE;
+    if (((uintptr_t)x[j] & 15) || ((uintptr_t)y[j] & 7) || (w_base[j] && ((uintptr_t)w_base[j] & 15))) return DZ_EALIGN;
+    n_total += N[j];
+  }
+  if (n_total > 0x7fffffff) return DZ_ESHAPE;
+  if (!workspace || workspace_bytes < dz_workspace_bytes(T, K, (int)n_total)) return DZ_EWORKSPACE;
+
+  hipStream_t st = (hipStream_t)stream;
+  int* perm = (int*)((char*)workspace + WS_HEADER) + 1024;
+  char* region = (char*)workspace + WS_HEADER + WS_PERM_BYTES;
+  MdlParams P[DZ_MAX_BATCH_CALLS];
+  for (int j = 0; j < ncalls; ++j) {
+    size_t cb, mb, sb;
+    dz_native_sizes(K, N[j], bits, group_size, &cb, &mb, &sb);
+    MdlParams& Q = P[j];
+    Q.x = (const _Float16*)x[j];
+    Q.wb = (const _Float16*)w_base[j];
+    Q.codes = (const u4_t*)codes_stacked[j];
+    Q.meta = (const u4_t*)meta_stacked[j];
+    Q.scales = (const _Float16*)scales_stacked[j];
+    Q.idx = (const long long*)indices;
+    Q.y = (_Float16*)y[j];
+    Q.status = (unsigned*)workspace;
+    Q.counters = (unsigned*)region;
+    region += ws_counter_bytes(N[j]);
+    Q.partials = (float*)region;
+    region += (size_t)MAX_KSPLIT * 32 * (size_t)N[j] * 4;
+    Q.codes_slot_u4 = (long long)(cb / 16);
+    Q.meta_slot_u4 = (long long)(mb / 16);
+    Q.scales_slot = (long long)(sb / 2);
+    Q.T = T; Q.K = K; Q.N = N[j]; Q.S = S; Q.gs = gs; Q.G = K / gs;
+    Q.accumulate = accumulate; Q.ldy = ldy[j];
+    Q.NP = N[j] / DZ_NPAIR; Q.NKB = K / DZ_KBLOCK;
+    Q.nsplit = 1; Q.cb = Q.NKB; Q.NPG = 0;
+    Q.perm = T <= 32 ? nullptr : perm;
+    Q.tok0 = 0;
+    Q.nchunk = 1;
+  }
+  const bool pre = !(bits == 2 && gs == K);
+  // 33..128 tokens: group the tokens by delta id on the device (no host round trip) and deal the
+  // groups to the chunks of 32; one launch carries all chunks
+  if (T > 32) hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
+  return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override);
 }
 
 int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
@@ -579,46 +643,9 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
                           size_t workspace_bytes, void* stream) {
   if (!x || !indices || !y) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
-  if (S < 1) return DZ_EINVAL;  // at least one slot: the kernels always address slot 0
-  size_t cb, mb, sb;
-  int rc = dz_native_sizes(K, N, bits, group_size, &cb, &mb, &sb);
-  if (rc) return rc;
-  int gs;
-  if ((rc = check_group(K, group_size, &gs))) return rc;
-  if (T < 1 || T > DZ_MAX_TOKENS_FUSED || ldy < N || ldy % 4) return DZ_ESHAPE;
-  if (((uintptr_t)x & 15) || ((uintptr_t)y & 7) || (w_base && ((uintptr_t)w_base & 15))) return DZ_EALIGN;
-  if (!workspace || workspace_bytes < dz_workspace_bytes(T, K, N)) return DZ_EWORKSPACE;
-
-  MdlParams P;
-  P.x = (const _Float16*)x;
-  P.wb = (const _Float16*)w_base;
-  P.codes = (const u4_t*)codes_stacked;
-  P.meta = (const u4_t*)meta_stacked;
-  P.scales = (const _Float16*)scales_stacked;
-  P.idx = (const long long*)indices;
-  P.y = (_Float16*)y;
-  P.status = (unsigned*)workspace;
-  int* seg_off = (int*)((char*)workspace + WS_HEADER);
-  int* perm = seg_off + 1024;
-  P.counters = (unsigned*)((char*)workspace + WS_HEADER + WS_PERM_BYTES);
-  P.partials = (float*)((char*)workspace + WS_HEADER + WS_PERM_BYTES + ws_counter_bytes(N));
-  P.codes_slot_u4 = (long long)(cb / 16);
-  P.meta_slot_u4 = (long long)(mb / 16);
-  P.scales_slot = (long long)(sb / 2);
-  P.T = T; P.K = K; P.N = N; P.S = S; P.gs = gs; P.G = K / gs;
-  P.accumulate = accumulate; P.ldy = ldy;
-  P.NP = N / DZ_NPAIR; P.NKB = K / DZ_KBLOCK;
-  P.nsplit = 1; P.cb = P.NKB; P.NPG = 0;
-  const bool pre = !(bits == 2 && gs == K);
-  hipStream_t st = (hipStream_t)stream;
-  P.perm = nullptr;
-  P.tok0 = 0;
-  if (T <= 32) return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
-  // 33..128 tokens: group the tokens by delta id on the device (no host round trip) and deal the
-  // groups to the chunks of 32; one launch carries all chunks
-  hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
-  P.perm = perm;
-  return dz_launch_mdl32(P, bits, pre, st, g_ksplit_override);
+  return dz_multi_delta_linear_batch(1, &x, &w_base, &codes_stacked, &meta_stacked, &scales_stacked, indices, &y,
+                                     &N, &ldy, T, K, S, bits, group_size, accumulate, workspace, workspace_bytes,
+                                     stream);
 }
 
 }  // extern "C"

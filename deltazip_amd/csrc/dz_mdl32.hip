@@ -25,13 +25,13 @@ namespace {
 
 constexpr int WK32 = 4;
 
+// The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
 template <int BITS, int TT, bool PRE, bool HAS_BASE>
-__global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
+__device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
+                                           unsigned char* smem, int& s_last) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? 4 : (TT == 2 ? 2 : 3);   // deltas per batch; two batches are in flight
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ int s_last;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform, in a scalar register
   const int jj = lane & 15, ga = lane >> 4;
@@ -39,15 +39,6 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   _Float16* xw = (_Float16*)smem + (size_t)wave * TP * DZ_KBLOCK;   // this wavefront's activations
   f4_t* red = (f4_t*)smem;                                          // reduction buffer, after the barrier
 
-  // workgroup -> (n-pair, k-chunk); the chunks of one n-pair are dealt to one XCD so that their
-  // partial sums can meet in that XCD's L2
-  // A launch may carry up to 4 chunks of 32 tokens (33..128 tokens, ordered by delta id): the
-  // workgroups of the chunks of one (n-pair, k-chunk) follow each other on the same XCD, so the
-  // base tile they all read comes from HBM once.
-  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-  const int per = P.nsplit * P.nchunk, rem = q % per;
-  const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
-  if (np >= P.NP) return;
   const int tok0 = P.tok0 + 32 * ch;
   const int Tc = min(32, P.T - 32 * ch);   // tokens of this chunk
   const int n0 = np * DZ_NPAIR;
@@ -417,49 +408,114 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   DZ_TS(9);
 }
 
-template <int BITS, int TT>
-int launch32(MdlParams P, bool pre, hipStream_t st, int ksplit_override) {
-  // K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
+// workgroup -> (n-pair, k-chunk, token chunk); the chunks of one n-pair are dealt to one XCD so
+// that their partial sums can meet in that XCD's L2.  A launch may carry up to 4 chunks of 32 tokens
+// (33..128 tokens, grouped by delta id): the workgroups of the chunks of one (n-pair, k-chunk)
+// follow each other on the same XCD, so the base tile they all read comes from HBM once.
+template <int BITS, int TT, bool PRE, bool HAS_BASE>
+__global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ int s_last;
+  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+  const int per = P.nsplit * P.nchunk, rem = q % per;
+  const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
+  if (np >= P.NP) return;
+  mdl32_body<BITS, TT, PRE, HAS_BASE>(P, np, kc, ch, smem, s_last);
+}
+
+// Several layer calls that share tokens, K and the slot table (the projections a fused layer
+// would hold in one weight: q/k/v, gate/up) in one launch: the n-pairs of the calls are numbered
+// through, a workgroup picks its call by its n-pair.  One call's tail (reduction, stores) then
+// overlaps the next one's loads instead of leaving the memory system idle between launches.
+template <int BITS, int TT, bool PRE, bool HAS_BASE>
+__global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlBatch B) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  __shared__ int s_last;
+  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+  const int per = B.p[0].nsplit * B.p[0].nchunk, rem = q % per;
+  const int npg = (q / per) * 8 + xcd, kc = rem / B.p[0].nchunk, ch = rem % B.p[0].nchunk;
+  if (npg >= B.np_end[DZ_MAX_BATCH - 1]) return;
+  // wavefront-uniform choice among the calls (np_end of unused entries repeats the total)
+  const int j = (npg >= B.np_end[0]) + (npg >= B.np_end[1]) + (npg >= B.np_end[2]);
+  const int first = j == 0 ? 0 : B.np_end[j - 1];
+  mdl32_body<BITS, TT, PRE, HAS_BASE>(B.p[j], npg - first, kc, ch, smem, s_last);
+}
+
+// K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
+static int choose_split(const MdlParams& P, int np_total, int ksplit_override) {
   int nsplit = ksplit_override;
   if (nsplit <= 0) {
     nsplit = 1;
     const int max_split = (P.NKB + WK32 - 1) / WK32;  // at least one round of 4 k-blocks each
-    while (nsplit < max_split && (long long)P.NP * nsplit * P.nchunk < 512) ++nsplit;
+    while (nsplit < max_split && (long long)np_total * nsplit * P.nchunk < 512) ++nsplit;
   }
   if (nsplit > 16 / P.nchunk) nsplit = 16 / P.nchunk;   // the workspace holds 16 sets of partial sums
   if (nsplit > P.NKB) nsplit = P.NKB;
-  P.cb = (P.NKB + nsplit - 1) / nsplit;
-  P.cb = (P.cb + WK32 - 1) / WK32 * WK32;  // whole rounds
-  P.nsplit = (P.NKB + P.cb - 1) / P.cb;
-  const int grid = (P.NP + 7) / 8 * 8 * P.nsplit * P.nchunk;
-  const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
-  static bool attr_done[4] = {false, false, false, false};
-  const bool has_base = P.wb != nullptr;
-  auto go = [&](auto kern, int slot) -> int {
-    if (!attr_done[slot]) {
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return DZ_ELAUNCH;
-      attr_done[slot] = true;
+  return nsplit;
+}
+
+template <int BITS, int TT>
+int launch32(MdlBatch B, int nprob, bool pre, hipStream_t st, int ksplit_override) {
+  // every call of a batch gets the split its n-pair count would get alone (the calls share K)
+  int np_min = B.p[0].NP;
+  for (int j = 1; j < nprob; ++j) np_min = B.p[j].NP < np_min ? B.p[j].NP : np_min;
+  const int nsplit0 = choose_split(B.p[0], np_min, ksplit_override);
+  int cb = (B.p[0].NKB + nsplit0 - 1) / nsplit0;
+  cb = (cb + WK32 - 1) / WK32 * WK32;  // whole rounds
+  const int nsplit = (B.p[0].NKB + cb - 1) / cb;
+  int np_total = 0;
+  bool has_base = B.p[0].wb != nullptr;
+  for (int j = 0; j < DZ_MAX_BATCH; ++j) {
+    if (j < nprob) {
+      B.p[j].cb = cb;
+      B.p[j].nsplit = nsplit;
+      np_total += B.p[j].NP;
+      if ((B.p[j].wb != nullptr) != has_base) return DZ_EINVAL;   // all with a base weight or none
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, P);
+    B.np_end[j] = np_total;
+  }
+  const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
+  const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
+  static bool attr_done[8] = {false, false, false, false, false, false, false, false};
+  auto go = [&](auto kern, auto bkern, int slot) -> int {
+    const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
+    const int which = slot + (nprob == 1 ? 0 : 4);
+    if (!attr_done[which]) {
+      if (hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return DZ_ELAUNCH;
+      attr_done[which] = true;
+    }
+    if (nprob == 1) hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, B.p[0]);
+    else hipLaunchKernelGGL(bkern, dim3(grid), dim3(64 * WK32), lds, st, B);
     return DZ_OK;
   };
   int rc;
-  if (pre) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, true, true>, 0) : go(dz_mdl32_kernel<BITS, TT, true, false>, 1);
-  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, false, true>, 2) : go(dz_mdl32_kernel<BITS, TT, false, false>, 3);
+  if (pre) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, true, true>, dz_mdl32_batch_kernel<BITS, TT, true, true>, 0)
+                         : go(dz_mdl32_kernel<BITS, TT, true, false>, dz_mdl32_batch_kernel<BITS, TT, true, false>, 1);
+  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, false, true>, dz_mdl32_batch_kernel<BITS, TT, false, true>, 2)
+                     : go(dz_mdl32_kernel<BITS, TT, false, false>, dz_mdl32_batch_kernel<BITS, TT, false, false>, 3);
   if (rc) return rc;
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
 }  // namespace
 
-// Launch of the T <= 32 kernel; called by dz_multi_delta_linear.
+// Launch of the fused kernel for one layer call or a batch of calls that share T, K, bits, the
+// scale grouping and the token order; called by dz_multi_delta_linear[_batch].
+int dz_launch_mdl32_batch(const MdlParams* P0, int nprob, int bits, bool pre, hipStream_t st, int ksplit_override) {
+  if (nprob < 1 || nprob > DZ_MAX_BATCH) return DZ_ESHAPE;
+  MdlBatch B;
+  for (int j = 0; j < DZ_MAX_BATCH; ++j) {
+    B.p[j] = P0[j < nprob ? j : 0];
+    B.p[j].nchunk = (P0[0].T + 31) / 32;
+  }
+  const int nchunk = B.p[0].nchunk, T = P0[0].T;
+  if (nchunk < 1 || nchunk > 4) return DZ_ESHAPE;
+  if (bits == 2) return T <= 16 ? launch32<2, 1>(B, nprob, pre, st, ksplit_override) : launch32<2, 2>(B, nprob, pre, st, ksplit_override);
+  return T <= 16 ? launch32<4, 1>(B, nprob, pre, st, ksplit_override) : launch32<4, 2>(B, nprob, pre, st, ksplit_override);
+}
+
 int dz_launch_mdl32(const MdlParams& P0, int bits, bool pre, hipStream_t st, int ksplit_override) {
-  MdlParams P = P0;
-  P.nchunk = (P.T + 31) / 32;
-  if (P.nchunk < 1 || P.nchunk > 4) return DZ_ESHAPE;
-  if (bits == 2) return P.T <= 16 ? launch32<2, 1>(P, pre, st, ksplit_override) : launch32<2, 2>(P, pre, st, ksplit_override);
-  return P.T <= 16 ? launch32<4, 1>(P, pre, st, ksplit_override) : launch32<4, 2>(P, pre, st, ksplit_override);
+  return dz_launch_mdl32_batch(&P0, 1, bits, pre, st, ksplit_override);
 }
 
 #ifdef DZ_TIMING

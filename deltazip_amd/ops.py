@@ -13,7 +13,7 @@ PyTorch is used for device memory and streams only; all arithmetic happens in th
 from __future__ import annotations
 
 import ctypes as C
-from typing import Dict, Optional, Tuple
+from typing import Dict, Optional, Sequence, Tuple
 
 import torch
 
@@ -360,6 +360,55 @@ def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: 
     bits = _bits_from_shapes(qweight_stacked, K, N)
     y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits)
     return y.view(*x.shape[:-1], N)
+
+
+def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked: Sequence[torch.Tensor],
+                      meta_stacked: Sequence[torch.Tensor], indices: torch.Tensor,
+                      base_weight: Sequence[torch.Tensor]):
+    """`apply_delta` for up to 4 projections that share the tokens -- q/k/v or gate/up held as
+    separate weights, which the reference fuses into one layer
+    (serving/vllm/delta/layers_marlin.py:281-487) -- in one launch.  `x` is one [T, K] tensor for
+    all or a sequence with one per projection; returns the list of [T, N_j] outputs."""
+    n = len(base_weight)
+    xs = [x] * n if isinstance(x, torch.Tensor) else list(x)
+    if not (len(xs) == len(qweight_stacked) == len(scales_stacked) == len(meta_stacked) == n) or not 1 <= n <= 4:
+        raise ValueError("one x / qweight / scales / meta / base weight per projection, at most 4 projections")
+    K = base_weight[0].shape[1]
+    T = xs[0].reshape(-1, K).shape[0]
+    bits = _bits_from_shapes(qweight_stacked[0], K, base_weight[0].shape[0])
+    G = scales_stacked[0][0].numel() // base_weight[0].shape[0]
+    S = qweight_stacked[0].shape[0]
+    if T > MAX_TOKENS_FUSED:
+        return [apply_delta(xs[j], qweight_stacked[j], scales_stacked[j], meta_stacked[j], indices, base_weight[j])
+                for j in range(n)]
+    _need_cuda(indices, *xs, *qweight_stacked, *scales_stacked, *meta_stacked, *base_weight)
+    if indices.dtype != torch.int64 or indices.numel() != T or not indices.is_contiguous():
+        raise ValueError("indices must be a contiguous int64 tensor with one entry per token")
+    group_size = -1 if G == 1 else K // G
+    x2s, outs, Ns = [], [], []
+    for j in range(n):
+        N = base_weight[j].shape[0]
+        x2 = xs[j].reshape(-1, K)
+        if (x2.dtype != torch.float16 or base_weight[j].dtype != torch.float16 or base_weight[j].shape[1] != K
+                or x2.shape[0] != T or not x2.is_contiguous() or not base_weight[j].is_contiguous()):
+            raise ValueError("x and base weights must be contiguous float16 with the same K and T")
+        cb, mb, sb = native_sizes(K, N, bits, group_size)
+        q, m, sc = qweight_stacked[j], meta_stacked[j], scales_stacked[j]
+        if (q.shape[0] != S or q[0].numel() * q.element_size() != cb or m[0].numel() * m.element_size() != mb
+                or sc[0].numel() * sc.element_size() != sb or sc.dtype != torch.float16
+                or not (q.is_contiguous() and m.is_contiguous() and sc.is_contiguous())):
+            raise ValueError("stacked delta tensors do not match the native layout for these sizes")
+        x2s.append(x2); Ns.append(N)
+        outs.append(torch.empty((T, N), dtype=torch.float16, device=x2.device))
+    vp = C.c_void_p * n
+    ptrs = lambda ts: vp(*[t.data_ptr() for t in ts])
+    ws = _workspace(x2s[0].device, T, K, sum(Ns))
+    rc = _lib.lib().dz_multi_delta_linear_batch(
+        n, ptrs(x2s), ptrs(base_weight), ptrs(qweight_stacked), ptrs(meta_stacked), ptrs(scales_stacked),
+        indices.data_ptr(), ptrs(outs), (C.c_int * n)(*Ns), (C.c_int * n)(*Ns), T, K, S, bits, group_size, 0,
+        ws.data_ptr(), ws.numel(), _stream())
+    _lib.check(rc, "dz_multi_delta_linear_batch")
+    return [outs[j].view(*xs[j].shape[:-1], Ns[j]) for j in range(n)]
 
 
 def add_delta(y: torch.Tensor, x: torch.Tensor, qweight: torch.Tensor, qzeros, scales: torch.Tensor,

@@ -41,6 +41,7 @@ extern "C" {
 #define DZ_EALIGN      -10   /* pointer not aligned as required                            */
 
 #define DZ_MAX_TOKENS_FUSED 128   /* largest T the fused decode kernel takes in one launch   */
+#define DZ_MAX_BATCH_CALLS 4      /* layer calls dz_multi_delta_linear_batch takes at once    */
 #define DZ_MAX_SLOTS_SEGMENT 768   /* largest S dz_segment takes (its tables live in LDS)      */
 #define DZ_MAX_SLOTS_MAP 4096      /* largest S dz_map_ids takes (the slot table lives in LDS) */
 
@@ -141,6 +142,21 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
                           int T, int K, int N, int S, int bits, int group_size,
                           int accumulate, int ldy, void* workspace, size_t workspace_bytes,
                           void* stream);
+
+/* Up to DZ_MAX_BATCH_CALLS layer calls in one launch: calls that share the tokens (T, indices),
+ * K, S, bits and group_size -- the projections the reference holds as one fused layer (q/k/v:
+ * MergedQKVParallelLinearWithDelta, gate/up: MergedColumnParallelLinearWithDelta,
+ * serving/vllm/delta/layers_marlin.py:281-487) when their weights are separate tensors.  Call j
+ * computes y[j][T, ldy[j]] (+)= x[j] @ w_base[j]^T + x[j] @ dequant(delta_j[indices])^T with
+ * N[j] output features, exactly as dz_multi_delta_linear would; in one launch the reduction and
+ * stores of one call overlap the loads of the next.  All calls have a base weight or none has.
+ * workspace: dz_workspace_bytes(T, K, N[0] + ... + N[ncalls-1]) bytes. */
+int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
+                                const void* const* codes_stacked, const void* const* meta_stacked,
+                                const void* const* scales_stacked, const int64_t* indices,
+                                uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
+                                int bits, int group_size, int accumulate, void* workspace,
+                                size_t workspace_bytes, void* stream);
 
 /* Dense fp16 GEMM on the matrix cores: y[T, ldy] (+)= x[T, K] @ w[N, K]^T, fp32 accumulation.
  * Stands in for the base product of LinearMethodBase.apply_weights

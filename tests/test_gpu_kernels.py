@@ -401,3 +401,32 @@ def test_compressor_argument_checks(dev):
         ops.compress_delta(torch.zeros(32, 200, device=dev), 4)
     with pytest.raises(ValueError):
         ops.compress_delta(torch.zeros(32, 256), 4)
+
+
+@pytest.mark.parametrize("bits,gs,t,ns", [(2, -1, 32, (128, 128, 128)), (4, 128, 7, (64, 256)), (2, -1, 64, (96, 32, 32, 160)),
+                                          (4, -1, 128, (64, 64))])
+def test_batched_calls_equal_separate_calls(dev, bits, gs, t, ns):
+    """Projections that share the tokens, in one launch: every output is bit for bit what the
+    separate call gives (same split of K, same order of additions), and matches the oracle."""
+    k, nd = 1024, 5
+    ps = [make_problem(n, k, bits, gs, nd, t, "uniform", 700 + 10 * j + n, dev) for j, n in enumerate(ns)]
+    ids = ps[0]["ids"]
+    ids_np = ps[0]["ids_np"]
+    x = ps[0]["x"]
+    ys = ops.apply_delta_batch(x, [p["q"] for p in ps], [p["s"] for p in ps], [p["m"] for p in ps], ids,
+                               [p["wb"] for p in ps])
+    torch.cuda.synchronize()
+    for p, y in zip(ps, ys):
+        sep = ops.apply_delta(x, p["q"], p["s"], p["m"], ids, p["wb"])
+        torch.cuda.synchronize()
+        assert torch.equal(y, sep)
+        ref = o.forward_ref(ps[0]["x_np"], p["wb_np"], p["dts"], ids_np)
+        assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+    # one x per projection
+    ys2 = ops.apply_delta_batch([p["x"] for p in ps], [p["q"] for p in ps], [p["s"] for p in ps],
+                                [p["m"] for p in ps], ids, [p["wb"] for p in ps])
+    torch.cuda.synchronize()
+    for p, y in zip(ps, ys2):
+        assert torch.equal(y, ops.apply_delta(p["x"], p["q"], p["s"], p["m"], ids, p["wb"]))
+    with pytest.raises(ValueError):
+        ops.apply_delta_batch(x, [ps[0]["q"]] * 5, [ps[0]["s"]] * 5, [ps[0]["m"]] * 5, ids, [ps[0]["wb"]] * 5)
