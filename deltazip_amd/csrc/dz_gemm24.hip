@@ -298,18 +298,21 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     const int pos = row_lo + wq * 64 + b * 16 + li;
     if (pos >= row_hi) continue;
     const int row = P.perm ? P.perm[pos] : pos;
+    _Float16* yrow = P.y + (size_t)row * P.ldy + n0 + wn * 128 + 4 * lg;
+    h4_t old[8];
+    if (P.accumulate) {
+      // all eight reads of the token's row in flight together
+#pragma unroll
+      for (int a = 0; a < 8; ++a)
+        old[a] = (n0 + wn * 128 + a * 16 + 4 * lg < P.N) ? *(const h4_t*)(yrow + a * 16) : (h4_t){0, 0, 0, 0};
+    }
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
-      const int n = n0 + wn * 128 + a * 16 + 4 * lg;
-      if (n >= P.N) continue;
+      if (n0 + wn * 128 + a * 16 + 4 * lg >= P.N) continue;
       f4_t v = acc[a][b];
-      _Float16* yp = P.y + (size_t)row * P.ldy + n;
-      if (P.accumulate) {
-        const h4_t o = *(const h4_t*)yp;
-        v += (f4_t){(float)o[0], (float)o[1], (float)o[2], (float)o[3]};
-      }
+      if (P.accumulate) v += (f4_t){(float)old[a][0], (float)old[a][1], (float)old[a][2], (float)old[a][3]};
       const h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-      *(h4_t*)yp = o;
+      *(h4_t*)(yrow + a * 16) = o;
     }
   }
 }

@@ -253,27 +253,30 @@ def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_id
 # ---------------------------------------------------------------------------------------------
 # workspace: zero-filled once per device, reused by every call on that device
 # ---------------------------------------------------------------------------------------------
-_workspaces: Dict[int, torch.Tensor] = {}
+# one per (device, stream): calls that share a workspace must be ordered on one stream
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, T: int, K: int, N: int) -> torch.Tensor:
     need = _lib.lib().dz_workspace_bytes(T, K, N)
     idx = device.index if device.index is not None else torch.cuda.current_device()
-    ws = _workspaces.get(idx)
+    key = (idx, _stream())
+    ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
         ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[idx] = ws
+        _workspaces[key] = ws
     return ws
 
 
 def workspace_status(device=None) -> int:
-    """Status word of the device workspace (bit 0: a delta id outside [-1, S) was seen and treated
-    as -1).  Synchronises; meant for debugging and tests."""
+    """Status words of the device's workspaces, OR-ed (bit 0: a delta id outside [-1, S) was seen
+    and treated as -1).  Synchronises; meant for debugging and tests."""
     idx = torch.cuda.current_device() if device is None else torch.device(device).index
-    ws = _workspaces.get(idx)
-    if ws is None:
-        return 0
-    return int(ws[:4].view(torch.int32).item())
+    status = 0
+    for (i, _), ws in _workspaces.items():
+        if i == idx:
+            status |= int(ws[:4].view(torch.int32).item())
+    return status
 
 
 # ---------------------------------------------------------------------------------------------

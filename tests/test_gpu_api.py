@@ -85,3 +85,25 @@ def test_row_parallel_rejects_bias_and_from_layer_passthrough(dev):
         layer(torch.zeros(4, 512, dtype=torch.float16, device=dev))
     act = torch.nn.ReLU()
     assert from_layer(act, 1, cfg, []) is act
+
+
+def test_two_streams_use_separate_workspaces(dev):
+    """The Python shim keeps one split-K workspace per (device, stream): calls issued on two streams
+    at the same time must not share partial sums."""
+    p1 = make_problem(256, 4096, 2, -1, 4, 32, "uniform", 11, dev)
+    p2 = make_problem(256, 4096, 2, -1, 4, 32, "uniform", 12, dev)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    outs = {1: [], 2: []}
+    for _ in range(8):
+        with torch.cuda.stream(s1):
+            outs[1].append(ops.apply_delta(p1["x"], p1["q"], p1["s"], p1["m"], p1["ids"], p1["wb"]))
+        with torch.cuda.stream(s2):
+            outs[2].append(ops.apply_delta(p2["x"], p2["q"], p2["s"], p2["m"], p2["ids"], p2["wb"]))
+    torch.cuda.synchronize()
+    for p, ys in ((p1, outs[1]), (p2, outs[2])):
+        ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+        for y in ys:
+            assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+            assert torch.equal(y, ys[0])
+    assert len({k for k in ops._workspaces if k[0] == dev.index}) >= 2
