@@ -17,6 +17,9 @@
  *   serving/vllm/delta/quant_linears/quant_linear_naive.py:35-96   QuantLinear.forward/from_tensors
  *   deltazip/nn_modules/qlinear_cuda.py:246-329    QuantLinear.unpack (dequantisation)
  *   deltazip/utils/converter.py:13-101             GPTQ layout -> kernel layout conversion
+ *   serving/vllm/delta/models.py:69-145            convert_mapping (delta id -> slot index tensors)
+ *   serving/vllm/delta/deltazip_marlin.py:21-86    per-delta embedding / output-projection tables
+ *   deltazip/core/quant.py, core/sparsegpt.py:55-66,123-135   quantiser and 2:4 mask of the compressor
  */
 #ifndef DZ_AMD_H
 #define DZ_AMD_H
