@@ -13,7 +13,7 @@ from .layers import (BaseLayerWithDelta, ColumnParallelLinearWithDelta, DeltaMap
                      from_layer_logits_processor)
 from .manager import DeltaModelManager, LRUCacheDeltaModelManager, create_delta_manager
 from .ops import (add_delta, add_delta_slice, apply_delta, apply_delta_batch, apply_delta_embed, apply_delta_uncompressed, compress_delta, dequant, merge, multi_delta_linear,
-                  native_sizes, repack_gptq_to_native, segment, stacked_shapes)
+                  native_sizes, repack_gptq_to_native, segment, stacked_shapes, token_order)
 from .quant_linear import QuantLinear
 
 __all__ = [
@@ -24,5 +24,5 @@ __all__ = [
     "repack_gptq_to_native", "segment", "stacked_shapes", "QuantLinear", "CompressionConfig",
     "DeltaLayerWeights", "DeltaModel", "convert_model", "compress_model", "DeltaModelManager", "LRUCacheDeltaModelManager",
     "create_delta_manager", "LogitsProcessorWithDelta", "VocabParallelEmbeddingWithDelta",
-    "from_layer_logits_processor", "apply_delta_embed", "apply_delta_uncompressed", "compress_delta", "apply_delta_batch",
+    "from_layer_logits_processor", "apply_delta_embed", "apply_delta_uncompressed", "compress_delta", "apply_delta_batch", "token_order",
 ]

@@ -27,7 +27,8 @@ SIGNATURES = {
     "dz_multi_delta_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_compress_2of4": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dz_multi_delta_linear_batch": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp,
-                                         C.c_size_t, _vp]),
+                                         _vp, C.c_size_t, _vp]),
+    "dz_token_order": (_i, [_vp, _i, _i, _vp, _vp]),
     "dz_map_ids": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "dz_workspace_bytes": (_sz, [_i, _i, _i]),
     "dz_multi_delta_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,

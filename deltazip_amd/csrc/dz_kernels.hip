@@ -577,8 +577,8 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
                                 const void* const* codes_stacked, const void* const* meta_stacked,
                                 const void* const* scales_stacked, const int64_t* indices,
                                 uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
-                                int bits, int group_size, int accumulate, void* workspace,
-                                size_t workspace_bytes, void* stream) {
+                                int bits, int group_size, int accumulate, const int32_t* order,
+                                void* workspace, size_t workspace_bytes, void* stream) {
   if (ncalls < 1 || ncalls > DZ_MAX_BATCH_CALLS) return DZ_ESHAPE;
   if (!x || !w_base || !codes_stacked || !meta_stacked || !scales_stacked || !indices || !y || !N || !ldy)
     return DZ_EINVAL;
@@ -625,15 +625,23 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     Q.accumulate = accumulate; Q.ldy = ldy[j];
     Q.NP = N[j] / DZ_NPAIR; Q.NKB = K / DZ_KBLOCK;
     Q.nsplit = 1; Q.cb = Q.NKB; Q.NPG = 0;
-    Q.perm = T <= 32 ? nullptr : perm;
+    Q.perm = T <= 32 ? nullptr : (order ? order : perm);
     Q.tok0 = 0;
     Q.nchunk = 1;
   }
   const bool pre = !(bits == 2 && gs == K);
   // 33..128 tokens: group the tokens by delta id on the device (no host round trip) and deal the
   // groups to the chunks of 32; one launch carries all chunks
-  if (T > 32) hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
+  if (T > 32 && !order)
+    hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
   return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override);
+}
+
+int dz_token_order(const int64_t* indices, int T, int S, int32_t* order, void* stream) {
+  if (!indices || !order) return DZ_EINVAL;
+  if (T < 1 || T > DZ_MAX_TOKENS_FUSED || S < 0) return DZ_ESHAPE;
+  hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, (hipStream_t)stream, (const long long*)indices, T, S, order);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
 int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
@@ -644,8 +652,8 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
   if (!x || !indices || !y) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
   return dz_multi_delta_linear_batch(1, &x, &w_base, &codes_stacked, &meta_stacked, &scales_stacked, indices, &y,
-                                     &N, &ldy, T, K, S, bits, group_size, accumulate, workspace, workspace_bytes,
-                                     stream);
+                                     &N, &ldy, T, K, S, bits, group_size, accumulate, nullptr, workspace,
+                                     workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -69,6 +69,7 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.base_layer = base_layer
         self.indices: Optional[torch.Tensor] = None
         self.indices_len: Optional[List[int]] = None
+        self.token_order: Optional[torch.Tensor] = None
 
     # -- state ---------------------------------------------------------------------------------
     def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
@@ -109,15 +110,21 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.meta_stacked[index].copy_(meta.view(self.meta_stacked[index].shape), non_blocking=ASYNC_COPY)
 
     def set_mapping(self, base_indices: torch.Tensor, sampler_indices=None, sampler_indices_padded=None,
-                    embeddings_indices=None, indices_len: Optional[List[int]] = None):
+                    embeddings_indices=None, indices_len: Optional[List[int]] = None,
+                    token_order: Optional[torch.Tensor] = None):
         # a view of the manager's buffer, re-read on the device at every call
         self.indices = base_indices
         self.indices_len = indices_len if indices_len is not None else [base_indices.numel()]
+        # optional: the manager's buffer with the order in which the kernel takes the tokens of a
+        # 33..128-token batch (the manager refreshes it with the mapping; None: computed per call)
+        self.token_order = token_order
 
     # -- compute -------------------------------------------------------------------------------
     def apply_weights(self, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        T = self.indices_len[0]
+        order = self.token_order[:T] if self.token_order is not None and 32 < T <= ops.MAX_TOKENS_FUSED else None
         return ops.apply_delta(x, self.qweight_stacked, self.scales_stacked, self.meta_stacked,
-                               self.indices[: self.indices_len[0]], self.base_layer.weight)
+                               self.indices[:T], self.base_layer.weight, order=order)
 
     def forward(self, input_):
         skip_bias_add = getattr(self.base_layer, "skip_bias_add", False)

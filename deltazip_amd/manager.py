@@ -28,7 +28,7 @@ import torch.nn as nn
 from . import ops
 from .checkpoint import DeltaModel
 from .config import DeltaConfig
-from .layers import BaseLayerWithDelta, DeltaMapping, from_layer, from_layer_logits_processor
+from .layers import BaseLayerWithDelta, DeltaMapping, LinearWithDelta, from_layer, from_layer_logits_processor
 
 
 class LRUCache:
@@ -119,6 +119,9 @@ class DeltaModelManager:
         self.sampler_indices = torch.empty(n, dtype=torch.long, device=self.device)
         self.sampler_indices_padded = torch.empty(n, dtype=torch.long, device=self.device)
         self.embeddings_indices = torch.empty(2, n, dtype=torch.long, device=self.device)
+        # order in which the fused kernel takes the tokens of a 33..128-token batch; refreshed with
+        # the mapping, shared by every linear layer
+        self.token_order = torch.zeros(ops.MAX_TOKENS_FUSED, dtype=torch.int32, device=self.device)
         # raw delta ids of the batch ([tokens | sampled rows]) and the id resident in each slot:
         # staged in pinned host memory, copied with one transfer each
         pin = self.device.type == "cuda"
@@ -256,6 +259,8 @@ class DeltaModelManager:
                     self.delta_slots + 1, self.vocab_size, self.delta_config.delta_extra_vocab_size,
                     self.base_indices, self.sampler_indices, self.sampler_indices_padded,
                     self.embeddings_indices)
+        if 32 < T <= ops.MAX_TOKENS_FUSED:
+            ops.token_order(self.base_indices[:T], self.delta_slots, out=self.token_order)
         # the layers keep a reference to this list
         self.indices_len[:] = (T, P, P, T)
 
@@ -289,8 +294,12 @@ class DeltaModelManager:
                 replace_submodule(self.model, module_name, new_module)
             self.register_module(module_name, new_module)
             self._register_packed_modules(module_name)
-            new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
-                                   self.embeddings_indices, self.indices_len)
+            if isinstance(new_module, LinearWithDelta):
+                new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
+                                       self.embeddings_indices, self.indices_len, token_order=self.token_order)
+            else:
+                new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
+                                       self.embeddings_indices, self.indices_len)
 
     def register_module(self, module_name: str, module: BaseLayerWithDelta) -> None:
         assert isinstance(module, BaseLayerWithDelta)

@@ -215,6 +215,23 @@ def compress_delta(delta: torch.Tensor, bits: int, group_size: int = -1):
     return q, m, s
 
 
+def token_order(indices: torch.Tensor, num_slots: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Order in which the fused kernel takes the tokens of a batch of up to 128 tokens (int32 [T]):
+    depends on the indices only, so it can be computed once per batch and passed to every layer
+    call of the step (`order=`), as the reference converts its mapping once per batch
+    (serving/vllm/delta/models.py:421-435)."""
+    _need_cuda(indices, out)
+    T = indices.numel()
+    if indices.dtype != torch.int64 or not indices.is_contiguous():
+        raise ValueError("indices must be a contiguous int64 tensor")
+    if out is None:
+        out = torch.empty(T, dtype=torch.int32, device=indices.device)
+    elif out.dtype != torch.int32 or out.numel() < T or not out.is_contiguous():
+        raise ValueError("out must be a contiguous int32 tensor with at least T entries")
+    _lib.check(_lib.lib().dz_token_order(indices.data_ptr(), T, num_slots, out.data_ptr(), _stream()), "dz_token_order")
+    return out[:T]
+
+
 def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_ids: torch.Tensor,
             max_deltas: int, vocab_size: int, extra_vocab_size: int, base_indices: torch.Tensor,
             sampler_indices: Optional[torch.Tensor] = None,
@@ -294,9 +311,11 @@ def _infer(qweight_stacked, scales_stacked, N: int):
 
 def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qweight_stacked,
                        scales_stacked, meta_stacked, indices: torch.Tensor, *, bits: int,
-                       out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+                       out: Optional[torch.Tensor] = None, accumulate: bool = False,
+                       order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ W_base^T + x @ dequant(delta[indices])^T.  `out` may be a column slice of a wider
-    tensor (last-dim stride 1); with accumulate=True the result is added to it."""
+    tensor (last-dim stride 1); with accumulate=True the result is added to it.  `order`: the
+    result of `token_order(indices, S)` when the caller already has it for this batch."""
     _need_cuda(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices)
     if x.dtype != torch.float16:
         raise ValueError("x must be float16")
@@ -338,11 +357,20 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
         return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
                                           indices, bits=bits, out=out, accumulate=accumulate)
     ws = _workspace(x.device, T, K, N)
-    rc = _lib.lib().dz_multi_delta_linear(
-        x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
-        qweight_stacked.data_ptr(), meta_stacked.data_ptr(), scales_stacked.data_ptr(),
-        indices.data_ptr(), out.data_ptr(), T, K, N, S, bits, group_size, 1 if accumulate else 0, ldy,
-        ws.data_ptr(), ws.numel(), _stream())
+    optr = _order_ptr(order, T, x.device)
+    if optr is None:
+        rc = _lib.lib().dz_multi_delta_linear(
+            x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
+            qweight_stacked.data_ptr(), meta_stacked.data_ptr(), scales_stacked.data_ptr(),
+            indices.data_ptr(), out.data_ptr(), T, K, N, S, bits, group_size, 1 if accumulate else 0, ldy,
+            ws.data_ptr(), ws.numel(), _stream())
+    else:
+        one = lambda p: (C.c_void_p * 1)(p)
+        rc = _lib.lib().dz_multi_delta_linear_batch(
+            1, one(x2.data_ptr()), one(base_weight.data_ptr() if base_weight is not None else None),
+            one(qweight_stacked.data_ptr()), one(meta_stacked.data_ptr()), one(scales_stacked.data_ptr()),
+            indices.data_ptr(), one(out.data_ptr()), (C.c_int * 1)(N), (C.c_int * 1)(ldy), T, K, S, bits, group_size,
+            1 if accumulate else 0, optr, ws.data_ptr(), ws.numel(), _stream())
     _lib.check(rc, "dz_multi_delta_linear")
     return out
 
@@ -356,22 +384,34 @@ def _bits_from_shapes(qweight_stacked: torch.Tensor, K: int, N: int) -> int:
 
 
 def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: torch.Tensor,
-                meta_stacked: torch.Tensor, indices: torch.Tensor, base_weight: torch.Tensor) -> torch.Tensor:
+                meta_stacked: torch.Tensor, indices: torch.Tensor, base_weight: torch.Tensor,
+                order: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Drop-in for serving/vllm/delta/deltazip_marlin.py:10-19.  Returns a new [T, N] tensor;
-    indices == -1 selects the base weight only."""
+    indices == -1 selects the base weight only.  (`order`: optional, see `token_order`.)"""
     N, K = base_weight.shape
     bits = _bits_from_shapes(qweight_stacked, K, N)
-    y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits)
+    y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits,
+                           order=order)
     return y.view(*x.shape[:-1], N)
+
+
+def _order_ptr(order: Optional[torch.Tensor], T: int, device) -> Optional[int]:
+    if order is None or T <= 32:
+        return None
+    if (not order.is_cuda or order.device != device or order.dtype != torch.int32 or order.numel() < T
+            or not order.is_contiguous()):
+        raise ValueError("order must be a contiguous int32 GPU tensor with one entry per token")
+    return order.data_ptr()
 
 
 def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked: Sequence[torch.Tensor],
                       meta_stacked: Sequence[torch.Tensor], indices: torch.Tensor,
-                      base_weight: Sequence[torch.Tensor]):
+                      base_weight: Sequence[torch.Tensor], order: Optional[torch.Tensor] = None):
     """`apply_delta` for up to 4 projections that share the tokens -- q/k/v or gate/up held as
     separate weights, which the reference fuses into one layer
     (serving/vllm/delta/layers_marlin.py:281-487) -- in one launch.  `x` is one [T, K] tensor for
-    all or a sequence with one per projection; returns the list of [T, N_j] outputs."""
+    all or a sequence with one per projection; `order` is what `token_order(indices, S)` returned
+    for this batch, if the caller has it; returns the list of [T, N_j] outputs."""
     n = len(base_weight)
     xs = [x] * n if isinstance(x, torch.Tensor) else list(x)
     if not (len(xs) == len(qweight_stacked) == len(scales_stacked) == len(meta_stacked) == n) or not 1 <= n <= 4:
@@ -409,7 +449,7 @@ def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked
     rc = _lib.lib().dz_multi_delta_linear_batch(
         n, ptrs(x2s), ptrs(base_weight), ptrs(qweight_stacked), ptrs(meta_stacked), ptrs(scales_stacked),
         indices.data_ptr(), ptrs(outs), (C.c_int * n)(*Ns), (C.c_int * n)(*Ns), T, K, S, bits, group_size, 0,
-        ws.data_ptr(), ws.numel(), _stream())
+        _order_ptr(order, T, indices.device), ws.data_ptr(), ws.numel(), _stream())
     _lib.check(rc, "dz_multi_delta_linear_batch")
     return [outs[j].view(*xs[j].shape[:-1], Ns[j]) for j in range(n)]
 

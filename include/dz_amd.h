@@ -153,13 +153,24 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
  * computes y[j][T, ldy[j]] (+)= x[j] @ w_base[j]^T + x[j] @ dequant(delta_j[indices])^T with
  * N[j] output features, exactly as dz_multi_delta_linear would; in one launch the reduction and
  * stores of one call overlap the loads of the next.  All calls have a base weight or none has.
- * workspace: dz_workspace_bytes(T, K, N[0] + ... + N[ncalls-1]) bytes. */
+ * order: NULL, or what dz_token_order wrote for these indices (then the grouping of the tokens is
+ * not repeated: the reference, too, converts the mapping once per batch and every layer reuses
+ * it, serving/vllm/delta/models.py:421-435).  workspace: dz_workspace_bytes(T, K, N[0] + ... +
+ * N[ncalls-1]) bytes. */
 int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
                                 const void* const* codes_stacked, const void* const* meta_stacked,
                                 const void* const* scales_stacked, const int64_t* indices,
                                 uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
-                                int bits, int group_size, int accumulate, void* workspace,
-                                size_t workspace_bytes, void* stream);
+                                int bits, int group_size, int accumulate, const int32_t* order,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/* The order in which the fused kernel takes the tokens of a batch of up to DZ_MAX_TOKENS_FUSED
+ * tokens, 32 per chunk: order[T], a permutation of 0..T-1 in which the tokens of one delta stay
+ * together and every chunk of 32 meets about the same number of distinct deltas.  Depends on the
+ * indices only, so one call serves every layer of a step (pass it as `order` above).  No
+ * counterpart in the reference beyond the scheduler's sort by delta id
+ * (serving/vllm/core/scheduler.py:101-104). */
+int dz_token_order(const int64_t* indices, int T, int S, int32_t* order, void* stream);
 
 /* Dense fp16 GEMM on the matrix cores: y[T, ldy] (+)= x[T, K] @ w[N, K]^T, fp32 accumulation.
  * Stands in for the base product of LinearMethodBase.apply_weights

@@ -430,3 +430,25 @@ def test_batched_calls_equal_separate_calls(dev, bits, gs, t, ns):
         assert torch.equal(y, ops.apply_delta(p["x"], p["q"], p["s"], p["m"], ids, p["wb"]))
     with pytest.raises(ValueError):
         ops.apply_delta_batch(x, [ps[0]["q"]] * 5, [ps[0]["s"]] * 5, [ps[0]["m"]] * 5, ids, [ps[0]["wb"]] * 5)
+
+
+@pytest.mark.parametrize("t,kind", [(33, "uniform"), (64, "zipf"), (128, "uniform"), (20, "uniform")])
+def test_token_order_is_a_permutation_and_reusable(dev, t, kind):
+    """dz_token_order: a permutation of the tokens in which every delta's tokens are contiguous; passing
+    it to the layer call gives bit for bit what the call computes with its own grouping."""
+    p = make_problem(64, 512, 4, -1, 12, t, kind, 808 + t, dev)
+    order = ops.token_order(p["ids"], 12)
+    torch.cuda.synchronize()
+    od = order.cpu().numpy()
+    assert sorted(od.tolist()) == list(range(t))
+    dealt = p["ids_np"][od]
+    if t > 32:
+        for c in range(0, t, 32):                      # inside a chunk every delta forms one run
+            ch = dealt[c:c + 32]
+            runs = 1 + int((ch[1:] != ch[:-1]).sum())
+            assert runs == len(set(ch.tolist()))
+    y0 = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"])
+    y1 = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], order=order)
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1)
+    assert o.rel_err(y1.cpu().numpy(), o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])) <= TOL
