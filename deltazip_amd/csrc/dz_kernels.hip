@@ -580,9 +580,11 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
                                 int bits, int group_size, int accumulate, const int32_t* order,
                                 void* workspace, size_t workspace_bytes, void* stream) {
   if (ncalls < 1 || ncalls > DZ_MAX_BATCH_CALLS) return DZ_ESHAPE;
-  if (!x || !w_base || !codes_stacked || !meta_stacked || !scales_stacked || !indices || !y || !N || !ldy)
-    return DZ_EINVAL;
-  if (S < 1) return DZ_EINVAL;  // at least one slot: the kernels always address slot 0
+  if (!x || !w_base || !indices || !y || !N || !ldy) return DZ_EINVAL;
+  if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
+  const void* const none[DZ_MAX_BATCH_CALLS] = {nullptr, nullptr, nullptr, nullptr};
+  if (S == 0) codes_stacked = meta_stacked = scales_stacked = none;
+  if (S < 0) return DZ_EINVAL;
   if (T < 1 || T > DZ_MAX_TOKENS_FUSED) return DZ_ESHAPE;
   int gs, rc;
   if ((rc = check_group(K, group_size, &gs))) return rc;
@@ -590,7 +592,9 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
   for (int j = 0; j < ncalls; ++j) {
     size_t cb, mb, sb;
     if ((rc = dz_native_sizes(K, N[j], bits, group_size, &cb, &mb, &sb))) return rc;
-    if (!x[j] || !y[j] || !codes_stacked[j] || !meta_stacked[j] || !scales_stacked[j]) return DZ_EINVAL;
+    if (!x[j] || !y[j]) return DZ_EINVAL;
+    // S = 0: a plain dense product with the base weight (every id counts as "no delta")
+    if (S == 0 ? !w_base[j] : (!codes_stacked[j] || !meta_stacked[j] || !scales_stacked[j])) return DZ_EINVAL;
     if (ldy[j] < N[j] || ldy[j] % 4) return DZ_ESHAPE;
     if (((uintptr_t)x[j] & 15) || ((uintptr_t)y[j] & 7) || (w_base[j] && ((uintptr_t)w_base[j] & 15))) return DZ_EALIGN;
     n_total += N[j];
@@ -608,9 +612,12 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     MdlParams& Q = P[j];
     Q.x = (const _Float16*)x[j];
     Q.wb = (const _Float16*)w_base[j];
-    Q.codes = (const u4_t*)codes_stacked[j];
-    Q.meta = (const u4_t*)meta_stacked[j];
-    Q.scales = (const _Float16*)scales_stacked[j];
+    // The kernel issues a fixed number of requests per round; those of absent deltas re-read 16
+    // bytes of slot 0.  Without slots they re-read the base weight instead (offsets stay inside
+    // it: a tile index times 1 or 2 KiB is below N*K/4 bytes, the weight has 2*N*K).
+    Q.codes = (const u4_t*)(S == 0 ? (const void*)w_base[j] : codes_stacked[j]);
+    Q.meta = (const u4_t*)(S == 0 ? (const void*)w_base[j] : meta_stacked[j]);
+    Q.scales = (const _Float16*)(S == 0 ? (const void*)w_base[j] : scales_stacked[j]);
     Q.idx = (const long long*)indices;
     Q.y = (_Float16*)y[j];
     Q.status = (unsigned*)workspace;
@@ -651,6 +658,7 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
                           size_t workspace_bytes, void* stream) {
   if (!x || !indices || !y) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
+  if (S == 0 && !w_base) return DZ_EINVAL;
   return dz_multi_delta_linear_batch(1, &x, &w_base, &codes_stacked, &meta_stacked, &scales_stacked, indices, &y,
                                      &N, &ldy, T, K, S, bits, group_size, accumulate, nullptr, workspace,
                                      workspace_bytes, stream);

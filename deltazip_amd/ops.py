@@ -157,9 +157,8 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     """Per-row dense product against the row's own full weight
     (serving/vllm/delta/deltazip_marlin.py:21-53, the lm_head of LogitsProcessorWithDelta):
     out[t] = x[t] @ delta_weights[indices[t]]^T, or x[t] @ base_embedding^T for indices[t] == -1.
-    The rows are grouped by id on the device and every group is one set of tiles of the grouped
-    matrix-core GEMM; like the reference's loop over torch.unique(indices), this reads the segment
-    sizes back to the host once."""
+    The rows are grouped by id on the device; like the reference's loop over
+    torch.unique(indices), this reads the group sizes back to the host once."""
     _need_cuda(x, delta_weights, indices, base_embedding)
     if x.dtype != torch.float16 or delta_weights.dtype != torch.float16 or base_embedding.dtype != torch.float16:
         raise ValueError("x and the weights must be float16")
@@ -175,21 +174,48 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     xs = x.index_select(0, perm64)
     ys = torch.empty((T, N), dtype=torch.float16, device=x.device)
     lib, st = _lib.lib(), _stream()
+    weight = lambda d: base_embedding if d < 0 else delta_weights[d]
+    segs = [(off[d + 1], off[d + 2], d) for d in range(-1, S) if off[d + 2] > off[d + 1]]
+    # A group of at most 128 rows is a decode-shaped, HBM-bound product: the fused kernel with no
+    # slots (a dense product with that group's weight) streams the weight once.  Larger groups go
+    # to the matrix-core GEMM, one launch for all of them.
+    small = [g for g in segs if g[1] - g[0] <= MAX_TOKENS_FUSED] if (K % 256 == 0 and N % 32 == 0) else []
+    large = [g for g in segs if g not in small]
+    if small:
+        none_ids = _minus_ones(x.device)
+        ws = _workspace(x.device, MAX_TOKENS_FUSED, K, N)
+        for lo, hi, d in small:
+            rc = lib.dz_multi_delta_linear(xs[lo:hi].data_ptr(), weight(d).data_ptr(), None, None, None,
+                                           none_ids.data_ptr(), ys[lo:hi].data_ptr(), hi - lo, K, N, 0, 2, -1, 0, N,
+                                           ws.data_ptr(), ws.numel(), st)
+            _lib.check(rc, "dz_multi_delta_linear")
+    if large:
+        blocks = lambda lo, hi, g: [(r, min(r + 256, hi), g, 0) for r in range(lo, hi, 256)]
 
-    def launch(w, w2, tiles):
-        tt = torch.tensor(tiles, dtype=torch.int32, device=x.device)
-        _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), w, w2, N * K, tt.data_ptr(), len(tiles), ys.data_ptr(),
-                                           T, K, N, 0, N, st), "dz_gemm_f16_grouped")
+        def launch(w, w2, tiles):
+            tt = torch.tensor(tiles, dtype=torch.int32, device=x.device)
+            _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), w, w2, N * K, tt.data_ptr(), len(tiles), ys.data_ptr(),
+                                               T, K, N, 0, N, st), "dz_gemm_f16_grouped")
 
-    blocks = lambda lo, hi, g: [(r, min(r + 256, hi), g, 0) for r in range(lo, hi, 256)]
-    if off[1] > off[0]:
-        launch(base_embedding.data_ptr(), None, blocks(off[0], off[1], -1))
-    tiles = [b for d in range(S) for b in blocks(off[d + 1], off[d + 2], d)]
-    if tiles:
-        launch(None, delta_weights.data_ptr(), tiles)
+        base_tiles = [b for lo, hi, d in large if d < 0 for b in blocks(lo, hi, -1)]
+        delta_tiles = [b for lo, hi, d in large if d >= 0 for b in blocks(lo, hi, d)]
+        if base_tiles:
+            launch(base_embedding.data_ptr(), None, base_tiles)
+        if delta_tiles:
+            launch(None, delta_weights.data_ptr(), delta_tiles)
     out = torch.empty_like(ys)
     out.index_copy_(0, perm64, ys)
     return out
+
+
+_minus_one_ids: Dict[int, torch.Tensor] = {}
+
+
+def _minus_ones(device) -> torch.Tensor:
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx not in _minus_one_ids:
+        _minus_one_ids[idx] = torch.full((MAX_TOKENS_FUSED,), -1, dtype=torch.int64, device=device)
+    return _minus_one_ids[idx]
 
 
 def compress_delta(delta: torch.Tensor, bits: int, group_size: int = -1):

@@ -135,6 +135,8 @@ size_t dz_workspace_bytes(int T, int K, int N);
  * indices [T] int64, -1 = base only, read on the device at execution time; y [T, ldy] fp16,
  * columns 0..N-1 written.  accumulate = 0: y = result; 1: y += result (fp32 add, one rounding).
  * Stands in for sbmm_4bit_2_4_native / ibmm_sparse_marlin at the call sites listed above.
+ * S = 0 (no slots; the delta pointers may then be NULL, w_base must not be): the dense product
+ * y (+)= x @ w_base^T alone, whatever the indices say.
  * Requires 1 <= T <= DZ_MAX_TOKENS_FUSED; above 32 tokens the tokens are grouped by id on the
  * device and handled 32 at a time, in one launch, the groups dealt so that every 32 meet about
  * the same number of deltas.  Larger batches are served by the host wrapper from dz_segment +

@@ -38,11 +38,15 @@ def test_argument_checks_happen_on_the_host(dzlib):
     ok = dict(T=4, K=512, N=64, S=2, bits=4, gs=-1, acc=0, ldy=64)
 
     def call(x=one, wb=one, q=one, m=one, s=one, idx=one, y=one, ws=one, wsb=1 << 30, **kw):
+        if kw.get("S") == 0 and "wsb" not in kw and wb is not None:
+            wsb = 16
         a = dict(ok); a.update(kw)
         return f(x, wb, q, m, s, idx, y, a["T"], a["K"], a["N"], a["S"], a["bits"], a["gs"], a["acc"], a["ldy"],
                  ws, wsb, None)
 
     assert call(x=None) == -1 and call(idx=None) == -1 and call(y=None) == -1 and call(q=None) == -1
+    assert call(S=0, q=None, m=None, s=None) == -8          # no slots: dense product only; next check is the workspace size
+    assert call(S=0, wb=None) == -1 and call(S=-1) == -1
     assert call(bits=3) == -3 and call(bits=8) == -3
     assert call(K=500) == -2 and call(N=48) == -2 and call(T=0) == -2 and call(T=129) == -2
     assert call(ldy=32) == -2 and call(ldy=66) == -2
