@@ -85,19 +85,37 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The 32 x 256 base tile: 16 loads of 16 bytes per lane.
+  // The 32 x 256 base tile: 16 loads of 16 bytes per lane.  One load covers 8 rows x 128 bytes
+  // (a request for 16 rows x 64 bytes moves 15 % fewer bytes per second on this memory system):
+  // lane (ga, jj) fetches row 16*s + 8*half + jj % 8, 16-byte chunk 2*ga + jj / 8 of the step's 128
+  // bytes.  The matrix instruction wants row jj in lane jj, so before use the upper eight lanes of
+  // each group of 16 trade places between the two halves (`base_operands`).
   auto issue_base = [&](int kb, int lane_r) {
     const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
-    const unsigned loff = (unsigned)(lane_r & 15) * Kb + (unsigned)(lane_r >> 4) * 16u;
+    const unsigned loff = (unsigned)(lane_r & 7) * Kb + (unsigned)(lane_r >> 4) * 32u + (unsigned)((lane_r >> 3) & 1) * 16u;
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
-      const char* ws = wbb + (size_t)(16 * s) * Kb;
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-          a[s][j][h] = __builtin_nontemporal_load((const u4_t*)(ws + loff + (128 * j + 64 * h)));
+        for (int h = 0; h < 2; ++h) {
+          const char* ws = wbb + (size_t)(16 * s + 8 * h) * Kb;
+          a[s][j][h] = __builtin_nontemporal_load((const u4_t*)(ws + loff + 128 * j));
+        }
     }
+  };
+  // u: row jj, chunk 2*ga of step j (lanes jj < 8 have it in the first half's register, lanes
+  // jj >= 8 take it from lane jj - 8 of the second half's); v: row jj, chunk 2*ga + 1.
+  auto base_operands = [&](const u4_t& ra, const u4_t& rb, h8_t& u, h8_t& v) {
+    H8U uu, vv;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      // row_ror:8 inside each group of 16 lanes; bank mask 0xC = lanes 8..15, 0x3 = lanes 0..7
+      uu.u[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)ra[d], (int)rb[d], 0x128, 0xF, 0xC, false);
+      vv.u[d] = (uint32_t)__builtin_amdgcn_update_dpp((int)rb[d], (int)ra[d], 0x128, 0xF, 0x3, false);
+    }
+    u = uu.h;
+    v = vv.h;
   };
 
   // token ids: lane t keeps the key of token t (0 = base only, id + 1 otherwise, INT_MAX for
@@ -276,15 +294,17 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
       for (int tt = 0; tt < TT; ++tt)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          h8_t blo, bhi;
-          ldsB(tt, j, blo, bhi);
+          // activations of chunks 2*ga and 2*ga + 1 of step j (the base operands' columns)
+          const char* px = (const char*)xw + (tt * 16 + jj) * (DZ_KBLOCK * 2) + (j >> 1) * 256;
+          const int c0 = (j & 1) * 8 + 2 * ga;
+          const h8_t blo = *(const h8_t*)(px + ((c0 ^ jj) << 4));
+          const h8_t bhi = *(const h8_t*)(px + (((c0 + 1) ^ jj) << 4));
 #pragma unroll
           for (int s = 0; s < 2; ++s) {
-            H8U a0, a1;
-            a0.v = a[s][j][0];
-            a1.v = a[s][j][1];
-            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0.h, blo, accb[s][tt], 0, 0, 0);
-            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1.h, bhi, accb[s][tt], 0, 0, 0);
+            h8_t u, v;
+            base_operands(a[s][j][0], a[s][j][1], u, v);
+            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(u, blo, accb[s][tt], 0, 0, 0);
+            accb[s][tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(v, bhi, accb[s][tt], 0, 0, 0);
           }
         }
     }
