@@ -74,6 +74,16 @@ __device__ __forceinline__ h8_t unpack4(uint32_t w, uint32_t MAGIC) {
   return r.h;
 }
 
+// Workgroup barrier without the memory fences of __syncthreads().  Those fences make the compiler
+// wait for every outstanding vector-memory request, which empties a ring of prefetched loads at
+// each barrier.  Callers order their LDS traffic themselves: an explicit s_waitcnt for LDS-direct
+// loads and LDS reads in front of the barrier.
+__device__ __forceinline__ void wg_barrier_nofence() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 struct MdlParams {
   const _Float16* x;
   const _Float16* wb;

@@ -222,7 +222,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     if (sd == 0 || sd + 1 >= nd) __builtin_amdgcn_s_waitcnt(0x0070);
     else if (sd + 2 >= nd) __builtin_amdgcn_s_waitcnt(0x0074);
     else __builtin_amdgcn_s_waitcnt(0x0078);
-    __syncthreads();
+    wg_barrier_nofence();   // __syncthreads() would wait for the whole ring
     if (sd == 0) {
       if (2 < nd) issue_xd(2);
       if (3 < nd) issue_xd(3);

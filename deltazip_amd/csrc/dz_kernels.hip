@@ -431,7 +431,12 @@ inline int check_group(int K, int group_size, int* gs_out) {
 }
 
 constexpr size_t WS_HEADER = 256;  // status word
-inline size_t ws_counter_bytes(int N) { return (((size_t)(N / DZ_NPAIR + 8) * 4 * 4) + 255) / 256 * 256; }   // 4 chunks
+// Arrival counters: a fixed area in front of the partial sums, 4 per n-pair (one per chunk of 32
+// tokens).  Its place must not depend on the sizes of a call: a counter is zero between launches
+// (the last workgroup to arrive resets it), and bytes that another call's partial sums have been
+// written to are not.
+constexpr size_t WS_COUNTER_BYTES = (size_t)1 << 20;
+constexpr long long WS_MAX_ROWS = (long long)(WS_COUNTER_BYTES / 16) * DZ_NPAIR;   // 2 M output rows per launch
 constexpr int MAX_KSPLIT = 16;
 constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // reserved + token order
 
@@ -565,12 +570,11 @@ int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size,
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
-// workspace: [status 256 B][token order][per call: arrival counters | partial sums]
-constexpr size_t WS_BATCH_SLACK = 4096;   // rounding of the per-call regions of a batch
+// workspace: [status 256 B][token order][arrival counters of all calls][per call: partial sums]
 size_t dz_workspace_bytes(int T, int K, int N) {
   (void)K;
   if (T < 1 || N < 1) return 0;
-  return WS_HEADER + WS_PERM_BYTES + ws_counter_bytes(N) + WS_BATCH_SLACK + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
+  return WS_HEADER + WS_PERM_BYTES + WS_COUNTER_BYTES + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
 }
 
 int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
@@ -599,12 +603,13 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     if (((uintptr_t)x[j] & 15) || ((uintptr_t)y[j] & 7) || (w_base[j] && ((uintptr_t)w_base[j] & 15))) return DZ_EALIGN;
     n_total += N[j];
   }
-  if (n_total > 0x7fffffff) return DZ_ESHAPE;
+  if (n_total > WS_MAX_ROWS) return DZ_ESHAPE;
   if (!workspace || workspace_bytes < dz_workspace_bytes(T, K, (int)n_total)) return DZ_EWORKSPACE;
 
   hipStream_t st = (hipStream_t)stream;
   int* perm = (int*)((char*)workspace + WS_HEADER) + 1024;
-  char* region = (char*)workspace + WS_HEADER + WS_PERM_BYTES;
+  unsigned* counters = (unsigned*)((char*)workspace + WS_HEADER + WS_PERM_BYTES);
+  char* region = (char*)workspace + WS_HEADER + WS_PERM_BYTES + WS_COUNTER_BYTES;
   MdlParams P[DZ_MAX_BATCH_CALLS];
   for (int j = 0; j < ncalls; ++j) {
     size_t cb, mb, sb;
@@ -621,8 +626,8 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     Q.idx = (const long long*)indices;
     Q.y = (_Float16*)y[j];
     Q.status = (unsigned*)workspace;
-    Q.counters = (unsigned*)region;
-    region += ws_counter_bytes(N[j]);
+    Q.counters = counters;
+    counters += (size_t)(N[j] / DZ_NPAIR) * 4;
     Q.partials = (float*)region;
     region += (size_t)MAX_KSPLIT * 32 * (size_t)N[j] * 4;
     Q.codes_slot_u4 = (long long)(cb / 16);

@@ -515,3 +515,4 @@ def add_delta_slice(y: torch.Tensor, x: torch.Tensor, qweight, qzeros, scales, g
 def set_ksplit(nsplit: int) -> None:
     """Benchmark hook: force the number of K chunks of the fused kernel (0 = automatic)."""
     _lib.lib().dz_set_ksplit(int(nsplit))
+

@@ -126,8 +126,9 @@ int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size,
                      void* out_meta, uint16_t* out_scales, float* scale_workspace, void* stream);
 
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
- * zero-filled once before first use; calls leave it ready for the next call.  Calls that share
- * a workspace must be ordered on one stream. */
+ * zero-filled once before first use; calls leave it ready for the next call (whatever their
+ * sizes: the arrival counters sit in a fixed 1 MiB area, which limits one launch to 2 M output
+ * rows in total).  Calls that share a workspace must be ordered on one stream. */
 size_t dz_workspace_bytes(int T, int K, int N);
 
 /* The layer.  x [T, K] fp16 row-major; w_base [N, K] fp16 row-major or NULL (delta only);

@@ -452,3 +452,28 @@ def test_token_order_is_a_permutation_and_reusable(dev, t, kind):
     torch.cuda.synchronize()
     assert torch.equal(y0, y1)
     assert o.rel_err(y1.cpu().numpy(), o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])) <= TOL
+
+
+
+def test_batched_calls_after_a_wide_single_call(dev):
+    """The arrival counters of a batch must not sit where an earlier, wider call kept partial sums:
+    a launch with three K chunks over 1024 rows (384 KiB of partial sums), then a batch whose
+    second call follows 128 rows; every result must still match the oracle."""
+    wide = make_problem(1024, 3072, 2, -1, 2, 31, "uniform", 41, dev)
+    try:
+        ops.set_ksplit(3)
+        ref = o.forward_ref(wide["x_np"], wide["wb_np"], wide["dts"], wide["ids_np"])
+        assert o.rel_err(run_layer(wide).cpu().numpy(), ref) <= TOL
+        ops.set_ksplit(4)
+        k, nd, t = 2048, 5, 32
+        ns = (128, 96, 32, 160)
+        ps = [make_problem(n, k, 2, -1, nd, t, "uniform", 900 + 10 * j + n, dev) for j, n in enumerate(ns)]
+        ids, x = ps[0]["ids"], ps[0]["x"]
+        ys = ops.apply_delta_batch(x, [p["q"] for p in ps], [p["s"] for p in ps], [p["m"] for p in ps], ids,
+                                   [p["wb"] for p in ps])
+        torch.cuda.synchronize()
+        for p, y in zip(ps, ys):
+            ref = o.forward_ref(ps[0]["x_np"], p["wb_np"], p["dts"], ps[0]["ids_np"])
+            assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+    finally:
+        ops.set_ksplit(0)
