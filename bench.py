@@ -36,7 +36,7 @@ T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1    # the default workload (configurati
 # HBM bytes per launch (average over the 4 launches of a step) of the default workload, from
 # rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what the same counter
 # reads for the --calib-copy-mib copy kernel; the figures are in profiles/*__hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 216875455
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 216410302
 
 
 def algorithmic_bytes(K, N, T, bits, d_present, G=1):
