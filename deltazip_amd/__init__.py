@@ -15,6 +15,7 @@ from .manager import DeltaModelManager, LRUCacheDeltaModelManager, create_delta_
 from .ops import (add_delta, add_delta_slice, apply_delta, apply_delta_batch, apply_delta_embed, apply_delta_uncompressed, compress_delta, dequant, merge, multi_delta_linear,
                   native_sizes, repack_gptq_to_native, segment, stacked_shapes, token_order)
 from .quant_linear import QuantLinear
+from .sparsegpt import Quantizer, SparseGPT
 
 __all__ = [
     "DeltaConfig", "BaseLayerWithDelta", "ColumnParallelLinearWithDelta", "DeltaMapping",
@@ -25,4 +26,5 @@ __all__ = [
     "DeltaLayerWeights", "DeltaModel", "convert_model", "compress_model", "DeltaModelManager", "LRUCacheDeltaModelManager",
     "create_delta_manager", "LogitsProcessorWithDelta", "VocabParallelEmbeddingWithDelta",
     "from_layer_logits_processor", "apply_delta_embed", "apply_delta_uncompressed", "compress_delta", "apply_delta_batch", "token_order",
+    "Quantizer", "SparseGPT",
 ]

@@ -260,17 +260,38 @@ def save_converted(tensors: Dict[str, torch.Tensor], compress_config: Compressio
 
 
 @torch.no_grad()
+def _compress_with_hessian(target: torch.Tensor, base: torch.Tensor, inputs: torch.Tensor,
+                           cfg: CompressionConfig):
+    """One module through SparseGPT with the reference's call sequence
+    (deltazip/modeling/_base.py:399-470): Hessian from the layer inputs, per-channel symmetric
+    quantizer, 2:4 sweep of target - base, native packing."""
+    from .sparsegpt import Quantizer, SparseGPT
+    layer = torch.nn.Linear(target.shape[1], target.shape[0], bias=False, dtype=target.dtype, device=target.device)
+    layer.weight.data = target.clone()
+    gpt = SparseGPT(layer)
+    gpt.quantizer = Quantizer()
+    gpt.quantizer.configure(cfg.bits, perchannel=True, sym=True, mse=False)
+    gpt.add_batch(inputs, None)
+    gpt.fasterprune(cfg.sparsity, prunen=cfg.prunen, prunem=cfg.prunem, percdamp=cfg.damp_percent, base_weight=base)
+    out = gpt.pack()
+    gpt.free()
+    return out
+
+
 def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: Dict[str, torch.Tensor],
                    compress_config: CompressionConfig, device="cuda:0",
-                   pack_modules: Optional[Dict[str, Tuple[str, int]]] = None) -> Dict[str, torch.Tensor]:
+                   pack_modules: Optional[Dict[str, Tuple[str, int]]] = None,
+                   calibration: Optional[Dict[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
     """Fine-tuned model + base model -> serving-layout state dict of the compressed delta (what
     `convert_model` makes of a checkpoint the reference's compressor wrote), on the GPU.
 
     Every 2-D `*.weight` outside UNCOMPRESSED_MODULES is compressed as the reference's per-layer
     step does it without calibration data: delta = target.float() - base.float()
     (deltazip/core/sparsegpt.py:55-62), scales from the un-pruned delta, 2:4 pruning by magnitude,
-    round-to-nearest codes (`ops.compress_delta`).  The Hessian-weighted error feedback of
-    SparseGPT (sparsegpt.py:69-146), which needs calibration activations, is not applied.  The
+    round-to-nearest codes (`ops.compress_delta`).  A module whose weight key appears in
+    `calibration` -- its layer inputs, [B, L, K] or [L, K], as the reference's compressor records them
+    layer by layer (deltazip/modeling/_base.py:261-576) -- goes through the Hessian-weighted sweep
+    with error feedback instead (`SparseGPT`, sparsegpt.py:27-146; per-channel scales only).  The
     remaining parameters are carried over from the fine-tuned model as they are, as the reference's
     command line tool saves them (cli/compress.py:134-152)."""
     if compress_config.bits not in (2, 4):
@@ -283,8 +304,14 @@ def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: 
     native: Dict[str, Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]] = {}
     for key, w in target_state_dict.items():
         if key.endswith(".weight") and w.dim() == 2 and not any(u in key for u in UNCOMPRESSED_MODULES):
-            delta = w.to(device).float() - base_state_dict[key].to(device).float()
-            q, m, s = ops.compress_delta(delta.contiguous(), bits, gs)
+            if calibration is not None and key in calibration:
+                if gs not in (-1, w.shape[1]):
+                    raise NotImplementedError("the Hessian-weighted sweep uses per-channel scales (group_size -1)")
+                q, m, s = _compress_with_hessian(w.to(device), base_state_dict[key].to(device),
+                                                 calibration[key].to(device), compress_config)
+            else:
+                delta = w.to(device).float() - base_state_dict[key].to(device).float()
+                q, m, s = ops.compress_delta(delta.contiguous(), bits, gs)
             native[key[: -len(".weight")]] = (q.cpu(), m.cpu(), s.cpu(), w.shape[1])
         elif key.endswith(".weight") and any(u in key for u in UNCOMPRESSED_MODULES):
             out[key[: -len(".weight")] + ".0.weight"] = w.detach().cpu()

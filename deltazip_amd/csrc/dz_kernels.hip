@@ -570,6 +570,39 @@ int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size,
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
+int dz_quant_scales(const float* delta, int K, int N, int bits, int group_size, float* scale32,
+                    uint16_t* scale16, void* stream) {
+  if (!delta || !scale32 || !scale16) return DZ_EINVAL;
+  int rc = dz_native_sizes(K, N, bits, group_size, nullptr, nullptr, nullptr);
+  if (rc) return rc;
+  int gs;
+  if ((rc = check_group(K, group_size, &gs))) return rc;
+  if ((uintptr_t)delta & 15) return DZ_EALIGN;
+  const int G = K / gs;
+  hipLaunchKernelGGL(dz_scales_kernel, dim3((unsigned)N * G), dim3(64), 0, (hipStream_t)stream, delta, K, N, gs, G,
+                     (float)((1 << bits) - 1), scale32, (_Float16*)scale16);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+int dz_pack_2of4(const float* w, const float* scale32, int K, int N, int bits, int group_size, void* out_codes,
+                 void* out_meta, void* stream) {
+  if (!w || !scale32 || !out_codes || !out_meta) return DZ_EINVAL;
+  int rc = dz_native_sizes(K, N, bits, group_size, nullptr, nullptr, nullptr);
+  if (rc) return rc;
+  int gs;
+  if ((rc = check_group(K, group_size, &gs))) return rc;
+  if ((uintptr_t)w & 15) return DZ_EALIGN;
+  const unsigned tiles = (unsigned)(N / DZ_NPAIR) * (K / DZ_KBLOCK);
+  hipStream_t st = (hipStream_t)stream;
+  if (bits == 2)
+    hipLaunchKernelGGL(dz_compress_kernel<2>, dim3(tiles), dim3(64), 0, st, w, scale32, K, N, gs,
+                       (uint32_t*)out_codes, (uint32_t*)out_meta);
+  else
+    hipLaunchKernelGGL(dz_compress_kernel<4>, dim3(tiles), dim3(64), 0, st, w, scale32, K, N, gs,
+                       (uint32_t*)out_codes, (uint32_t*)out_meta);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
 // workspace: [status 256 B][token order][arrival counters of all calls][per call: partial sums]
 size_t dz_workspace_bytes(int T, int K, int N) {
   (void)K;

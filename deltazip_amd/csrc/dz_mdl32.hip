@@ -119,7 +119,8 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   };
 
   // token ids: lane t keeps the key of token t (0 = base only, id + 1 otherwise, INT_MAX for
-  // padding lanes); mdelta marks the tokens that carry a delta.  Both are set in round 0.
+  // padding lanes); mdelta marks the tokens that carry a delta.  Both are set in the first pass
+  // of the loop over k-blocks.
   int key = 0x7fffffff;
   unsigned long long mdelta = 0;
   // The ids are requested before anything else and nothing more is requested until they are in:

@@ -13,6 +13,7 @@ PyTorch is used for device memory and streams only; all arithmetic happens in th
 from __future__ import annotations
 
 import ctypes as C
+import math
 from typing import Dict, Optional, Sequence, Tuple
 
 import torch
@@ -239,6 +240,76 @@ def compress_delta(delta: torch.Tensor, bits: int, group_size: int = -1):
                                      s.data_ptr(), ws.data_ptr(), _stream())
     _lib.check(rc, "dz_compress_2of4")
     return q, m, s
+
+
+def quant_scales(delta: torch.Tensor, bits: int, group_size: int = -1):
+    """Symmetric scales of the reference's Quantizer.find_params (deltazip/core/quant.py:48-130,
+    perchannel, sym) for an fp32 delta [N, K] on the GPU: (scale32 [G, N] fp32, scale16 [G, N] fp16)."""
+    _need_cuda(delta)
+    if delta.dtype != torch.float32 or delta.dim() != 2 or not delta.is_contiguous():
+        raise ValueError("delta must be a contiguous float32 [N, K] tensor")
+    N, K = delta.shape
+    _, _, ss = stacked_shapes(K, N, bits, group_size)
+    s32 = torch.empty(ss, dtype=torch.float32, device=delta.device)
+    s16 = torch.empty(ss, dtype=torch.float16, device=delta.device)
+    rc = _lib.lib().dz_quant_scales(delta.data_ptr(), K, N, bits, group_size, s32.data_ptr(), s16.data_ptr(), _stream())
+    _lib.check(rc, "dz_quant_scales")
+    return s32, s16
+
+
+def pack_2of4(w: torch.Tensor, scale32: torch.Tensor, bits: int, group_size: int = -1):
+    """(qweight, meta) of one slot in the native layout from fp32 values [N, K] that are 2:4 sparse and
+    on the grid of `scale32` [G, N] (what `obs_sweep` leaves behind)."""
+    _need_cuda(w, scale32)
+    if w.dtype != torch.float32 or w.dim() != 2 or not w.is_contiguous():
+        raise ValueError("w must be a contiguous float32 [N, K] tensor")
+    N, K = w.shape
+    qs, ms, ss = stacked_shapes(K, N, bits, group_size)
+    if scale32.dtype != torch.float32 or tuple(scale32.shape) != tuple(ss) or not scale32.is_contiguous():
+        raise ValueError("scale32 must be a contiguous float32 [G, N] tensor")
+    q = torch.empty(qs, dtype=torch.int32, device=w.device)
+    m = torch.empty(ms, dtype=torch.int16, device=w.device)
+    rc = _lib.lib().dz_pack_2of4(w.data_ptr(), scale32.data_ptr(), K, N, bits, group_size, q.data_ptr(), m.data_ptr(),
+                                 _stream())
+    _lib.check(rc, "dz_pack_2of4")
+    return q, m
+
+
+def hessian_add(H: torch.Tensor, x: torch.Tensor, nsamples: int, batch: int) -> int:
+    """H <- H * n/(n+b) + (sqrt(2/(n+b)) x)^T (sqrt(2/(n+b)) x) in place for x [T, K] (fp16 or fp32),
+    as SparseGPT.add_batch does for a linear layer (deltazip/core/sparsegpt.py:27-40); returns n + b."""
+    _need_cuda(H, x)
+    K = H.shape[0]
+    if H.dtype != torch.float32 or tuple(H.shape) != (K, K) or not H.is_contiguous():
+        raise ValueError("H must be a contiguous float32 [K, K] tensor")
+    if x.dim() != 2 or x.shape[1] != K or x.dtype not in (torch.float16, torch.float32) or not x.is_contiguous():
+        raise ValueError("x must be a contiguous [T, K] float16 or float32 tensor")
+    n = nsamples + batch
+    rc = _lib.lib().dz_hessian_add(H.data_ptr(), x.data_ptr(), int(x.dtype == torch.float16), x.shape[0], K,
+                                   float(nsamples / n), math.sqrt(2.0 / n), _stream())
+    _lib.check(rc, "dz_hessian_add")
+    return n
+
+
+def obs_sweep(W: torch.Tensor, hinv_upper: torch.Tensor, scale: Optional[torch.Tensor], bits: int = 4,
+              prunen: int = 2, prunem: int = 4) -> torch.Tensor:
+    """The column sweep of SparseGPT.fasterprune (deltazip/core/sparsegpt.py:92-146) over W [N, K] fp32
+    in place: n:m pruning by w^2 / diag(hinv)^2, rounding to the grid of `scale` [N] (None: no
+    rounding), error compensation along the rows of `hinv_upper`.  Returns the per-row losses [N]."""
+    _need_cuda(W, hinv_upper, scale)
+    N, K = W.shape
+    if W.dtype != torch.float32 or not W.is_contiguous():
+        raise ValueError("W must be a contiguous float32 [N, K] tensor")
+    if hinv_upper.dtype != torch.float32 or tuple(hinv_upper.shape) != (K, K) or not hinv_upper.is_contiguous():
+        raise ValueError("hinv_upper must be a contiguous float32 [K, K] tensor")
+    if scale is not None and (scale.dtype != torch.float32 or scale.numel() != N or not scale.is_contiguous()):
+        raise ValueError("scale must be a contiguous float32 tensor with one entry per row")
+    err = torch.empty((N, 128), dtype=torch.float32, device=W.device)
+    loss = torch.zeros(N, dtype=torch.float32, device=W.device)
+    rc = _lib.lib().dz_obs_sweep(W.data_ptr(), hinv_upper.data_ptr(), scale.data_ptr() if scale is not None else None,
+                                 N, K, bits, prunen, prunem, err.data_ptr(), loss.data_ptr(), _stream())
+    _lib.check(rc, "dz_obs_sweep")
+    return loss
 
 
 def token_order(indices: torch.Tensor, num_slots: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -120,10 +120,41 @@ int dz_embedding_select(const int64_t* tokens, const int64_t* indices, const uin
  * q = clamp(rint(x / scale) + 2^(bits-1), 0, 2^bits - 1) with the fp32 scale (quant.py:9-18),
  * stored scale = fp16(scale) (qlinear_cuda.py:153-156).  The result equals, byte for byte, what
  * dz_repack_2of4 makes of the same delta compressed and packed the reference's way.  The
- * Hessian-weighted solve of SparseGPT (sparsegpt.py:69-146) is not part of this.
+ * Hessian-weighted sweep of SparseGPT is dz_obs_sweep below.
  * scale_workspace: G * N floats of device memory (G = K / group_size, 1 for -1). */
 int dz_compress_2of4(const float* delta, int K, int N, int bits, int group_size, void* out_codes,
                      void* out_meta, uint16_t* out_scales, float* scale_workspace, void* stream);
+
+/* The two halves of dz_compress_2of4 on their own.  dz_quant_scales: the symmetric scales of
+ * Quantizer.find_params (deltazip/core/quant.py:48-130, perchannel, sym) as fp32 [G, N] and fp16
+ * [G, N].  dz_pack_2of4: codes and positions in the native layout from values that are already
+ * 2:4 sparse and on the grid of the given fp32 scales (what dz_obs_sweep leaves in W); other
+ * values are pruned by magnitude and rounded as in dz_compress_2of4. */
+int dz_quant_scales(const float* delta, int K, int N, int bits, int group_size, float* scale32,
+                    uint16_t* scale16, void* stream);
+int dz_pack_2of4(const float* w, const float* scale32, int K, int N, int bits, int group_size, void* out_codes,
+                 void* out_meta, void* stream);
+
+/* Layer Hessian of SparseGPT.add_batch (deltazip/core/sparsegpt.py:27-40):
+ * H <- H * scale_h + (scale_x * x)^T (scale_x * x) for x [T, K] (fp16 if x_is_fp16, else fp32),
+ * H [K, K] fp32; the caller passes scale_h = n / (n + b) and scale_x = sqrt(2 / (n + b)) for b new
+ * samples after n.  The sum over tokens runs in ascending order, one rounding per operation.
+ * K % 64 == 0. */
+int dz_hessian_add(float* H, const void* x, int x_is_fp16, int T, int K, float scale_h, float scale_x,
+                   void* stream);
+
+/* The sweep of SparseGPT.fasterprune (deltazip/core/sparsegpt.py:92-146) over W [N, K] fp32 in
+ * place, in blocks of 128 columns: in every aligned group of prunem columns the prunen columns
+ * with the smallest w^2 / diag(hinv)^2 are set to 0 (ties keep the lower column; prunen = 0: no
+ * pruning), every column is rounded to the grid scale[row] * (q - 2^(bits-1)), q in [0, 2^bits)
+ * (scale = NULL: not rounded), and its error, divided by the diagonal, is subtracted from the
+ * columns to its right along the row of hinv_upper -- the upper Cholesky factor of the inverse of
+ * the dampened Hessian (sparsegpt.py:80-84), [K, K] fp32 row-major.  loss [N] += the row's
+ * sum of (w - q)^2 / diag^2 / 2 per block.  err_workspace: N * 128 floats.  Sums run in
+ * ascending column order with one rounding per operation, so the result equals a plain fp32
+ * restatement with that order bit for bit.  K % 128 == 0, prunem <= 8 and a divisor of 64. */
+int dz_obs_sweep(float* W, const float* hinv_upper, const float* scale, int N, int K, int bits, int prunen,
+                 int prunem, float* err_workspace, float* loss, void* stream);
 
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
  * zero-filled once before first use; calls leave it ready for the next call (whatever their

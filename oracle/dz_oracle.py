@@ -18,6 +18,11 @@ Pinning status (what independent evidence each function is checked against in te
   convert_mapping_ref           hand-computed index tensors for small batches          (pinned)
   embed_select_ref, linear_select_ref   plain row selection / torch CPU matmul per row, checked
                                 against hand-built tables                              (pinned)
+  hessian_add_batch_ref, hinv_upper_ref, obs_sweep_ref   float64 Gram matrix, identity-Hessian
+                                reduction to the pinned quantizer, closed-form surgeon update,
+                                first-order optimality of unvisited columns (pinned by mathematics;
+                                the reference's matmul summation order and topk tie order are
+                                undefined: "parity unpinned" against it on those two points)
 The fused third-party kernel the reference calls on the serving path (triteia
 `sbmm_4bit_2_4_native`, un-vendored and un-pinned: scripts/install.sh:2, call site
 serving/vllm/delta/deltazip_marlin.py:18) cannot be inspected: its bit layout and rounding are
@@ -490,3 +495,103 @@ def make_ids(kind, t, n_deltas, seed):
     if kind == "blocks":
         return np.repeat(np.arange(n_deltas), t // n_deltas).astype(np.int64)
     raise ValueError(kind)
+
+
+# --------------------------------------------------------------------------------------
+# f-4: the Hessian-aware sweep (deltazip/core/sparsegpt.py:25-146), n:m pruning with error
+# compensation.  Pinned by what the mathematics fixes (tests/test_oracle_obs.py): an identity
+# Hessian reduces it to prune_2of4_magnitude + quantize; without quantisation every kept weight to
+# the right of the sweep satisfies the first-order optimality condition (W0 - W) H[:, todo] = 0;
+# pruning one weight of a 1 x K row equals the closed-form optimal-brain-surgeon update.  The
+# floating-point summation order of the reference's matmuls and torch.topk's tie order are not
+# defined by the reference: here sums run in ascending index order with one rounding per operation
+# and ties keep the lower column ("parity unpinned" against the reference for those two points).
+# --------------------------------------------------------------------------------------
+
+
+def hessian_add_batch_ref(H: np.ndarray, nsamples: int, inp: np.ndarray):
+    """sparsegpt.py:27-40 for a linear layer: inp [B, L, K] (or [L, K] = one sample).
+    H <- H * n/(n+B); inp <- sqrt(2/(n+B)) * inp; H <- H + inp^T inp.  Returns (H, n+B)."""
+    x = np.asarray(inp, dtype=np.float32)
+    b = 1 if x.ndim == 2 else x.shape[0]
+    x = x.reshape(-1, x.shape[-1])
+    H = (H.astype(np.float32) * np.float32(nsamples / (nsamples + b))).astype(np.float32)
+    n = nsamples + b
+    xs = (np.float32(np.sqrt(2.0 / n)) * x).astype(np.float32)
+    acc = np.zeros_like(H)
+    for t in range(xs.shape[0]):                       # ascending token order, one rounding per op
+        acc = (acc + (xs[t][:, None] * xs[t][None, :]).astype(np.float32)).astype(np.float32)
+    return (H + acc).astype(np.float32), n
+
+
+def hinv_upper_ref(H: np.ndarray, W: np.ndarray, percdamp: float = 0.01):
+    """sparsegpt.py:69-84: dead columns, dampening, H^-1 through Cholesky, its upper factor.
+    Returns (Hinv_upper [K, K] fp32, W with dead columns zeroed).  torch CPU LAPACK in fp32."""
+    H = torch.from_numpy(np.array(H, dtype=np.float32))
+    W = np.array(W, dtype=np.float32)
+    dead = torch.diag(H) == 0
+    H[dead, dead] = 1
+    W[:, dead.numpy()] = 0
+    damp = percdamp * torch.mean(torch.diag(H))
+    idx = torch.arange(H.shape[0])
+    H[idx, idx] += damp
+    H = torch.linalg.cholesky(H)
+    H = torch.cholesky_inverse(H)
+    H = torch.linalg.cholesky(H, upper=True)
+    return np.ascontiguousarray(H.numpy()), W
+
+
+def obs_sweep_ref(W: np.ndarray, hinv: np.ndarray, scale=None, bits: int = 4, prunen: int = 2,
+                  prunem: int = 4, blocksize: int = 128, stop: int = None):
+    """sparsegpt.py:92-146.  W [N, K] fp32, hinv = upper Cholesky factor of H^-1, scale [N] fp32
+    (per-row symmetric scale, zero = 2^(bits-1)) or None for pruning without quantisation.
+    Returns (W_out [N, K], losses [N]); columns >= `stop` (a multiple of blocksize) are left as
+    the sweep has updated them so far (used by the optimality test)."""
+    W = np.array(W, dtype=np.float32)
+    n, k = W.shape
+    hinv = np.asarray(hinv, dtype=np.float32)
+    maxq = np.float32(2**bits - 1)
+    zero = np.float32(2 ** (bits - 1))
+    losses = np.zeros(n, dtype=np.float32)
+    stop = k if stop is None else stop
+    for i1 in range(0, stop, blocksize):
+        i2 = min(i1 + blocksize, k)
+        count = i2 - i1
+        W1 = W[:, i1:i2].copy()
+        Q1 = np.zeros_like(W1)
+        Err1 = np.zeros_like(W1)
+        H1 = hinv[i1:i2, i1:i2]
+        dg = np.diag(H1).astype(np.float32)
+        mask1 = np.zeros(W1.shape, dtype=bool)
+        lsum = np.zeros(n, dtype=np.float32)
+        for i in range(count):
+            w = W1[:, i].copy()
+            d = dg[i]
+            if prunen != 0 and i % prunem == 0:
+                tmp = (W1[:, i:i + prunem] ** 2).astype(np.float32) / (dg[i:i + prunem] ** 2).astype(np.float32)[None, :]
+                # keep the (prunem - prunen) largest; ties keep the lower column
+                m = tmp.shape[1]
+                rank = np.zeros(tmp.shape, dtype=np.int8)
+                for a in range(m):
+                    for b in range(m):
+                        if a != b:
+                            rank[:, a] += (tmp[:, b] > tmp[:, a]) if b > a else (tmp[:, b] >= tmp[:, a])
+                mask1[:, i:i + prunem] = rank >= (m - prunen)
+            q = np.where(mask1[:, i], np.float32(0), w).astype(np.float32)
+            if scale is not None:
+                sc = scale.astype(np.float32)
+                q = (sc * (np.clip(np.rint(q / sc) + zero, 0, maxq) - zero)).astype(np.float32)
+            Q1[:, i] = q
+            diff = (w - q).astype(np.float32)
+            lsum = (lsum + ((diff * diff).astype(np.float32) / np.float32(d * d)).astype(np.float32)).astype(np.float32)
+            err = (diff / d).astype(np.float32)
+            W1[:, i:] = (W1[:, i:] - (err[:, None] * H1[i, i:][None, :]).astype(np.float32)).astype(np.float32)
+            Err1[:, i] = err
+        W[:, i1:i2] = Q1
+        losses = (losses + lsum / np.float32(2)).astype(np.float32)
+        if i2 < k:
+            acc = np.zeros((n, k - i2), dtype=np.float32)
+            for j in range(count):                      # ascending, one rounding per operation
+                acc = (acc + (Err1[:, j][:, None] * hinv[i1 + j, i2:][None, :]).astype(np.float32)).astype(np.float32)
+            W[:, i2:] = (W[:, i2:] - acc).astype(np.float32)
+    return W, losses

@@ -69,6 +69,25 @@ def test_argument_checks_happen_on_the_host(dzlib):
     assert dzlib.dz_gemm_f16(None, one, one, 8, 128, 128, 0, 128, None) == -1
 
 
+def test_compressor_entry_points_check_their_arguments(dzlib):
+    one = C.c_void_p(0x1000)   # never dereferenced
+    assert dzlib.dz_hessian_add(None, one, 1, 8, 256, 0.5, 0.5, None) == -1
+    assert dzlib.dz_hessian_add(one, one, 1, 0, 256, 0.5, 0.5, None) == -2
+    assert dzlib.dz_hessian_add(one, one, 1, 8, 100, 0.5, 0.5, None) == -2
+    sweep = lambda **kw: dzlib.dz_obs_sweep(kw.get("W", one), one, kw.get("scale", one), kw.get("N", 32), kw.get("K", 256),
+                                            kw.get("bits", 4), kw.get("pn", 2), kw.get("pm", 4), one, one, None)
+    assert sweep(W=None) == -1
+    assert sweep(K=192) == -2                    # whole blocks of 128 columns
+    assert sweep(bits=5) == -3
+    assert sweep(pn=2, pm=3) == -2               # group size must divide 64
+    assert sweep(pn=4, pm=4) == -2
+    assert sweep(pn=2, pm=16) == -2
+    assert dzlib.dz_quant_scales(one, 256, 32, 3, -1, one, one, None) == -3
+    assert dzlib.dz_quant_scales(one, 256, 32, 4, 100, one, one, None) == -4
+    assert dzlib.dz_pack_2of4(one, None, 256, 32, 4, -1, one, one, None) == -1
+    assert dzlib.dz_pack_2of4(one, one, 250, 32, 4, -1, one, one, None) == -2
+
+
 def test_python_wrappers_refuse_cpu_tensors(dzlib):
     import torch
     from deltazip_amd import ops, QuantLinear, DeltaConfig

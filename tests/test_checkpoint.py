@@ -182,3 +182,42 @@ def test_compress_model_on_gpu(dev, bits, gs):
     assert dm.get_delta("model.layers.0.self_attn.qkv_proj")._compressed and not dm.get_delta("lm_head")._compressed
     with pytest.raises(NotImplementedError):
         ck.compress_model(base, target, ck.CompressionConfig(bits=4, prunen=0, prunem=0), device=dev)
+
+
+@pytest.mark.gpu
+def test_compress_model_with_calibration_inputs(dev):
+    """A module listed in `calibration` takes the Hessian-weighted path: its packed delta equals what
+    the oracle's sweep gives for the same inputs, the others stay on the magnitude path."""
+    g = torch.Generator().manual_seed(12)
+    n, k = 64, 256
+    keys = ["model.layers.0.self_attn.o_proj.weight", "model.layers.0.mlp.down_proj.weight"]
+    base = {key: (torch.randn(n, k, generator=g) * 0.02).half() for key in keys}
+    target = {key: (base[key].float() + torch.randn(n, k, generator=g) * 1e-2).half() for key in keys}
+    x = torch.randn(4, 128, k, generator=g)
+    x = (x + 0.5 * torch.roll(x, 1, dims=2)).half()
+    cfg = ck.CompressionConfig(bits=4, sparsity=0.5, prunen=2, prunem=4)
+    out = ck.compress_model(base, target, cfg, device=dev, calibration={keys[0]: x})
+    # oracle for the calibrated module
+    d32 = target[keys[0]].float().numpy() - base[keys[0]].float().numpy()
+    H, _ = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, x.numpy())
+    hinv, W0 = o.hinv_upper_ref(H, d32)
+    scale, zero = o.find_params_sym(d32, 4)
+    # the factor comes from the GPU's Cholesky in the product: compare through the compensated error
+    want, _ = o.obs_sweep_ref(W0, hinv, scale[:, 0], 4)
+    q, m, s = (out[f"model.layers.0.self_attn.o_proj.0.{t}"] for t in ("qweight", "meta", "scales"))
+    got = native_dequant(q, m, s, k, 4).astype(np.float32)
+    xf = x.float().numpy().reshape(-1, k)
+    e_got = np.linalg.norm((d32 - got) @ xf.T)
+    e_want = np.linalg.norm((d32 - want) @ xf.T)
+    plain = o.quantize(np.where(o.prune_2of4_magnitude(d32), d32, np.float32(0)), scale, zero, 15)
+    e_plain = np.linalg.norm((d32 - plain) @ xf.T)
+    assert abs(e_got - e_want) <= 0.02 * e_want and e_got < 0.95 * e_plain
+    # same integer codes, up to the few roundings that flip with the last bits of the GPU's factor
+    s16 = s.numpy().astype(np.float32).reshape(-1, 1)
+    assert (np.rint(got / s16) != np.rint(want / scale)).mean() < 0.02
+    # the other module: magnitude path, bit for bit
+    d2 = target[keys[1]].float().numpy() - base[keys[1]].float().numpy()
+    codes, scales16, zeros, _ = o.compress_delta(d2, 4, -1)
+    qw, qz, sc, gi = o.pack_codes_gptq(codes, zeros, scales16, 4)
+    q2, m2, s2 = (out[f"model.layers.0.mlp.down_proj.0.{t}"] for t in ("qweight", "meta", "scales"))
+    assert np.array_equal(native_dequant(q2, m2, s2, k, 4), o.dequant_gptq(qw, qz, sc, gi, 4).T)

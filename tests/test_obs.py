@@ -1,0 +1,116 @@
+"""Hessian-aware compression on the GPU (dz_hessian_add, dz_obs_sweep, dz_quant_scales,
+dz_pack_2of4 through the C ABI) against the oracle's restatement of
+deltazip/core/sparsegpt.py:25-146: bit for bit, since both sum in the same order."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import dz_oracle as o
+from deltazip_amd import ops
+from deltazip_amd.sparsegpt import Quantizer, SparseGPT
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(n, k, tokens, seed):
+    rng = np.random.default_rng(seed)
+    W = (rng.standard_normal((n, k)) * 0.01).astype(np.float32)
+    X = rng.standard_normal((tokens, k)).astype(np.float32)
+    X = (X + 0.5 * np.roll(X, 1, axis=1)).astype(np.float16)       # layer inputs are fp16
+    return W, X
+
+
+def test_hessian_add_bit_exact(dev):
+    k = 256
+    _, xa = _inputs(4, k, 3 * 40, 1)
+    _, xb = _inputs(4, k, 77, 2)
+    H = torch.zeros(k, k, dtype=torch.float32, device=dev)
+    n = ops.hessian_add(H, torch.from_numpy(xa).to(dev), 0, 3)            # 3 samples of 40 tokens
+    n = ops.hessian_add(H, torch.from_numpy(xb).float().to(dev), n, 1)    # one more, passed as fp32
+    torch.cuda.synchronize()
+    Href, nref = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, xa.reshape(3, 40, k))
+    Href, nref = o.hessian_add_batch_ref(Href, nref, xb)
+    assert n == nref == 4
+    assert np.array_equal(H.cpu().numpy(), Href)
+
+
+@pytest.mark.parametrize("n,k,bits,quant,prune", [(32, 256, 4, True, True), (64, 384, 2, True, True),
+                                                  (32, 256, 4, False, True), (40, 256, 4, True, False)])
+def test_obs_sweep_bit_exact(dev, n, k, bits, quant, prune):
+    W, X = _inputs(n, k, 1024, 10 + n + k + bits)
+    H, _ = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, X)
+    hinv, W0 = o.hinv_upper_ref(H, W)
+    scale, _ = o.find_params_sym(W, bits)
+    sc = scale[:, 0].copy() if quant else None
+    pn, pm = (2, 4) if prune else (0, 0)
+    want, want_loss = o.obs_sweep_ref(W0, hinv, sc, bits, pn, pm)
+    Wd = torch.from_numpy(W0.copy()).to(dev)
+    loss = ops.obs_sweep(Wd, torch.from_numpy(hinv).to(dev), torch.from_numpy(sc).to(dev) if quant else None,
+                         bits, pn, pm)
+    torch.cuda.synchronize()
+    assert np.array_equal(Wd.cpu().numpy(), want)
+    assert np.array_equal(loss.cpu().numpy(), want_loss)
+
+
+def test_scales_and_pack_match_the_reference_pipeline(dev):
+    """Values on the grid with two zeros per group of four -> the same native bytes as compressing
+    and packing the reference's way (oracle) and converting with the repacker."""
+    n, k, bits = 64, 512, 4
+    W, X = _inputs(n, k, 512, 3)
+    s32, s16 = ops.quant_scales(torch.from_numpy(W).to(dev), bits)
+    scale, zero = o.find_params_sym(W, bits)
+    assert np.array_equal(s32.cpu().numpy()[0], scale[:, 0])
+    assert np.array_equal(s16.cpu().numpy()[0].view(np.uint16), scale[:, 0].astype(np.float16).view(np.uint16))
+    H, _ = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, X)
+    hinv, W0 = o.hinv_upper_ref(H, W)
+    out, _ = o.obs_sweep_ref(W0, hinv, scale[:, 0], bits)
+    q, m = ops.pack_2of4(torch.from_numpy(out).to(dev), s32, bits)
+    torch.cuda.synchronize()
+    codes = o.quantize_codes(out, scale, zero, 2**bits - 1)                    # [N, K]
+    qw, qz, sc16, gi = o.pack_codes_gptq(np.ascontiguousarray(codes.T), zero.T.astype(np.int32),
+                                         scale.T.astype(np.float16), bits)
+    rq, rm, rs = ops.repack_gptq_to_native(torch.from_numpy(qw), torch.from_numpy(qz), torch.from_numpy(sc16),
+                                           torch.from_numpy(gi), bits)
+    assert torch.equal(q.cpu(), rq) and torch.equal(m.cpu(), rm)
+    # and the packed delta dequantises to the swept values rounded to fp16 the reference's way
+    dq = ops.dequant(q, m, s16, k, n, bits).cpu().numpy()
+    assert np.array_equal(dq, o.dequant_gptq(qw, qz, sc16, gi, bits).T)
+
+
+def test_sparsegpt_interface_end_to_end(dev):
+    """SparseGPT(layer).add_batch / fasterprune / pack with the reference's call sequence
+    (deltazip/modeling/_base.py:399-470): the layer ends up holding base + compressed delta, the
+    compensation lowers the layer's output error below plain magnitude pruning + rounding."""
+    n, k, bits = 64, 256, 4
+    rng = np.random.default_rng(7)
+    base = (rng.standard_normal((n, k)) * 0.02).astype(np.float16)
+    delta, X = _inputs(n, k, 2048, 8)
+    target = (base.astype(np.float32) + delta).astype(np.float16)
+    layer = torch.nn.Linear(k, n, bias=False, dtype=torch.float16, device=dev)
+    layer.weight.data = torch.from_numpy(target).to(dev)
+    gpt = SparseGPT(layer)
+    gpt.quantizer = Quantizer()
+    gpt.quantizer.configure(bits, perchannel=True, sym=True, mse=False)
+    xs = torch.from_numpy(X).to(dev)
+    for i in range(0, 2048, 512):
+        gpt.add_batch(xs[i:i + 512].reshape(4, 128, k), None)
+    assert gpt.nsamples == 16
+    scale, zero, g_idx, avg_loss, Wc = gpt.fasterprune(0.5, prunen=2, prunem=4, base_weight=torch.from_numpy(base).to(dev))
+    torch.cuda.synchronize()
+    assert tuple(scale.shape) == (n, 1) and float(zero[0, 0]) == 8 and int(g_idx.abs().sum()) == 0 and avg_loss > 0
+    d32 = target.astype(np.float32) - base.astype(np.float32)
+    got = Wc.float().cpu().numpy()
+    assert ((got.reshape(n, -1, 4) == 0).sum(axis=2) >= 2).all()
+    sc, zr = o.find_params_sym(d32, bits)
+    plain = o.quantize(np.where(o.prune_2of4_magnitude(d32), d32, np.float32(0)), sc, zr, 15)
+    xf = X.astype(np.float32)
+    assert np.linalg.norm((d32 - got) @ xf.T) < 0.95 * np.linalg.norm((d32 - plain) @ xf.T)
+    assert torch.equal(layer.weight.data, (Wc + torch.from_numpy(base).to(dev)).half())
+    q, m, s16 = gpt.pack()
+    dq = ops.dequant(q, m, s16, k, n, bits).float().cpu().numpy()
+    assert np.allclose(dq, got, rtol=2e-3, atol=1e-7)
+    gpt.free()
+    with pytest.raises(NotImplementedError):
+        SparseGPT(layer).fasterprune(0.5)                       # unstructured sparsity
+    with pytest.raises(NotImplementedError):
+        SparseGPT(layer).fasterprune(0.0, actorder=True)
