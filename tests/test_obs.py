@@ -34,15 +34,19 @@ def test_hessian_add_bit_exact(dev):
     assert np.array_equal(H.cpu().numpy(), Href)
 
 
-@pytest.mark.parametrize("n,k,bits,quant,prune", [(32, 256, 4, True, True), (64, 384, 2, True, True),
-                                                  (32, 256, 4, False, True), (40, 256, 4, True, False)])
+@pytest.mark.parametrize("n,k,bits,quant,prune", [(32, 256, 4, True, (2, 4)), (64, 384, 2, True, (2, 4)),
+                                                  (32, 256, 4, False, (2, 4)), (40, 256, 4, True, (0, 0)),
+                                                  (32, 256, 4, True, (4, 8)), (33, 128, 2, True, (1, 2)),
+                                                  (256, 1024, 4, True, (2, 4))])
 def test_obs_sweep_bit_exact(dev, n, k, bits, quant, prune):
     W, X = _inputs(n, k, 1024, 10 + n + k + bits)
-    H, _ = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, X)
+    H, _ = o.hessian_add_batch_ref(np.zeros((k, k), np.float32), 0, X[:256] if k > 512 else X)
+    if k > 512:
+        H = H + np.eye(k, dtype=np.float32)                 # fewer samples than columns: keep it well conditioned
     hinv, W0 = o.hinv_upper_ref(H, W)
     scale, _ = o.find_params_sym(W, bits)
     sc = scale[:, 0].copy() if quant else None
-    pn, pm = (2, 4) if prune else (0, 0)
+    pn, pm = prune
     want, want_loss = o.obs_sweep_ref(W0, hinv, sc, bits, pn, pm)
     Wd = torch.from_numpy(W0.copy()).to(dev)
     loss = ops.obs_sweep(Wd, torch.from_numpy(hinv).to(dev), torch.from_numpy(sc).to(dev) if quant else None,
