@@ -48,6 +48,23 @@ class Quantizer:
         return self.scale is not None
 
 
+def _inverse_hessian_factor(H: torch.Tensor, W: torch.Tensor, percdamp: float) -> torch.Tensor:
+    """sparsegpt.py:69-84, in place on H and W: input columns that never fired get a unit diagonal and
+    a zero weight column, the diagonal is raised by percdamp times its mean, and the upper Cholesky
+    factor of the inverse comes back (the sweep reads its rows).  The factorisations are torch.linalg
+    calls on the device the Hessian lives on."""
+    d = torch.diagonal(H)                      # a view: writes go to H
+    dead = d == 0
+    d[dead] = 1
+    W[:, dead] = 0
+    d += percdamp * torch.mean(d)
+    lower = torch.linalg.cholesky(H)
+    hinv = torch.linalg.cholesky(torch.cholesky_inverse(lower), upper=True)
+    if bool(torch.isnan(hinv).any()):
+        raise ValueError("Hinv contains nan, aborting...")
+    return hinv.contiguous()
+
+
 class SparseGPT:
     def __init__(self, layer: nn.Linear):
         if not isinstance(layer, nn.Linear):
@@ -91,22 +108,11 @@ class SparseGPT:
         quantizer = getattr(self, "quantizer", None)
         if quantizer is not None and not quantizer.ready():
             quantizer.find_params(W, weight=True)
-        H = self.H
-        del self.H
-        dead = torch.diag(H) == 0
-        H[dead, dead] = 1
-        W[:, dead] = 0
-        damp = percdamp * torch.mean(torch.diag(H))
-        diag = torch.arange(self.columns, device=self.dev)
-        H[diag, diag] += damp
-        H = torch.linalg.cholesky(H)
-        H = torch.cholesky_inverse(H)
-        H = torch.linalg.cholesky(H, upper=True)
-        if bool(torch.isnan(H).any()):
-            raise ValueError("Hinv contains nan, aborting...")
+        hinv = _inverse_hessian_factor(self.H, W, percdamp)
+        self.H = None
         W = W.contiguous()
         scale = quantizer.scale.reshape(-1).contiguous() if quantizer is not None else None
-        losses = ops.obs_sweep(W, H.contiguous(), scale, quantizer.bits if quantizer is not None else 4,
+        losses = ops.obs_sweep(W, hinv, scale, quantizer.bits if quantizer is not None else 4,
                                prunen, prunem)
         g_idx = torch.zeros(self.columns, dtype=torch.int32, device=self.dev)     # i // columns
         self._packed_from = W
