@@ -25,18 +25,33 @@ HIPCC_FLAGS = [
 
 
 def build_library(verbose: bool = False, extra_flags=()) -> str:
+    """Compiles every source (one hipcc process each, side by side) and links libdz_amd.so."""
+    from concurrent.futures import ThreadPoolExecutor
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
-    srcs = [os.path.join(CSRC, s) for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-x", "hip", *srcs, "-o", LIB]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, capture_output=True, text=True)
-    # hipcc's host pass reports that it does not know the packed-fp32 feature; that is expected
-    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + err)
-    if verbose and err.strip():
-        print(err, file=sys.stderr)
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        # hipcc's host pass reports that it does not know the packed-fp32 feature; that is expected
+        err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + err)
+        if verbose and err.strip():
+            print(err, file=sys.stderr)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
+        run([hipcc, *[f for f in HIPCC_FLAGS if f != "-shared"], *extra_flags, "-x", "hip", "-c",
+             os.path.join(CSRC, src), "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(len(srcs), os.cpu_count() or 4)) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB])
     return LIB
 
 

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "dz_layout.h"
 
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
@@ -17,7 +19,7 @@ typedef uint32_t u2_t __attribute__((ext_vector_type(2)));
 // Phase timestamps for kernel tuning; compiled out unless DZ_TIMING is defined.
 #ifdef DZ_TIMING
 static __device__ unsigned long long* g_dz_ts;
-#define DZ_TS(i) do { if (lane == 0) { g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + (i)] = clock64(); if ((i) == 0) g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + 14] = wall_clock64(); if ((i) == 9) g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + 15] = wall_clock64(); } } while (0)
+#define DZ_TS(i) do { if (lane == 0) g_dz_ts[((size_t)blockIdx.x * 16 + wave) * 16 + (i)] = wall_clock64(); } while (0)
 #else
 #define DZ_TS(i) do { } while (0)
 #endif
@@ -93,7 +95,6 @@ struct MdlParams {
   const long long* idx;
   _Float16* y;
   float* partials;
-  unsigned* counters;
   unsigned* status;
   const int* perm;   // token order (rows of x / y / idx) or nullptr: rows tok0, tok0 + 1, ...
   int tok0;          // first position of this launch in that order; T counts from there
@@ -138,6 +139,19 @@ __device__ __forceinline__ Frag<BITS> load_frag(const MdlParams& P, int d, int n
     f.code[BITS == 2 ? 0 : 1] = __builtin_nontemporal_load((const u4_t*)(cb + lo + 1024));
   }
   return f;
+}
+
+// Raises a kernel's dynamic-LDS limit once per device (the attribute belongs to the device's copy
+// of the kernel).  `done` holds one bit per device; two threads that meet here at the same time
+// both set the attribute, which is harmless.
+inline bool dz_lds_limit_once(std::atomic<unsigned long long>& done, const void* kernel, int bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) return false;
+  const unsigned long long bit = 1ull << dev;
+  if (done.load(std::memory_order_acquire) & bit) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
 }
 
 // Launch of the T <= 32 kernel (dz_mdl32.hip).

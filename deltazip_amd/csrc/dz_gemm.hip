@@ -16,6 +16,7 @@
 #include <stdint.h>
 
 #include "../../include/dz_amd.h"
+#include "dz_device.h"
 
 typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
 typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
@@ -189,12 +190,8 @@ int gemm_launch(GemmParams P, int ntiles_m, void* stream) {
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
   const size_t lds = 2 * 2 * SLAB;
-  static bool attr_done = false;
-  if (!attr_done) {
-    if (hipFuncSetAttribute((const void*)dz_gemm_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return DZ_ELAUNCH;
-    attr_done = true;
-  }
+  static std::atomic<unsigned long long> attr_done{0};
+  if (!dz_lds_limit_once(attr_done, (const void*)dz_gemm_kernel, (int)lds)) return DZ_ELAUNCH;
   hipLaunchKernelGGL(dz_gemm_kernel, dim3(grid), dim3(256), lds, (hipStream_t)stream, P);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }

@@ -376,13 +376,9 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
   const size_t lds = 4 * SLAB + 8 * 3072;   // two base buffers = four ring stages, + staged k-block
-  static bool attr_done[2] = {false, false};
+  static std::atomic<unsigned long long> attr_done[2];
   auto go = [&](auto kern, int which) -> int {
-    if (!attr_done[which]) {
-      if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-        return DZ_ELAUNCH;
-      attr_done[which] = true;
-    }
+    if (!dz_lds_limit_once(attr_done[which], (const void*)kern, (int)lds)) return DZ_ELAUNCH;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(512), lds, (hipStream_t)stream, P);
     return DZ_OK;
   };

@@ -8,6 +8,8 @@
 #include <stdint.h>
 
 #include "../../include/dz_amd.h"
+#include <atomic>
+
 #include "dz_device.h"
 
 namespace {
@@ -421,7 +423,7 @@ __global__ __launch_bounds__(128) void dz_deal_kernel(const long long* __restric
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-int g_ksplit_override = 0;
+std::atomic<int> g_ksplit_override{0};
 
 inline int check_group(int K, int group_size, int* gs_out) {
   int gs = (group_size == -1 || group_size == K) ? K : group_size;
@@ -431,12 +433,6 @@ inline int check_group(int K, int group_size, int* gs_out) {
 }
 
 constexpr size_t WS_HEADER = 256;  // status word
-// Arrival counters: a fixed area in front of the partial sums, 4 per n-pair (one per chunk of 32
-// tokens).  Its place must not depend on the sizes of a call: a counter is zero between launches
-// (the last workgroup to arrive resets it), and bytes that another call's partial sums have been
-// written to are not.
-constexpr size_t WS_COUNTER_BYTES = (size_t)1 << 20;
-constexpr long long WS_MAX_ROWS = (long long)(WS_COUNTER_BYTES / 16) * DZ_NPAIR;   // 2 M output rows per launch
 constexpr int MAX_KSPLIT = 16;
 constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // reserved + token order
 
@@ -467,7 +463,7 @@ const char* dz_strerror(int code) {
   }
 }
 
-void dz_set_ksplit(int nsplit) { g_ksplit_override = nsplit; }
+void dz_set_ksplit(int nsplit) { g_ksplit_override.store(nsplit, std::memory_order_relaxed); }
 
 int dz_dequant(const void* codes, const void* meta, const void* scales, int K, int N, int bits,
                int group_size, uint16_t* out, void* stream) {
@@ -603,11 +599,13 @@ int dz_pack_2of4(const float* w, const float* scale32, int K, int N, int bits, i
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
-// workspace: [status 256 B][token order][arrival counters of all calls][per call: partial sums]
+// workspace: [status 256 B][token order][per call: partial sums].  The partial-sum slots are
+// their own "ready" marks (all zero bits = empty) and every launch leaves them empty again, so the
+// workspace is zero-filled once by its owner and never again.
 size_t dz_workspace_bytes(int T, int K, int N) {
   (void)K;
   if (T < 1 || N < 1) return 0;
-  return WS_HEADER + WS_PERM_BYTES + WS_COUNTER_BYTES + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
+  return WS_HEADER + WS_PERM_BYTES + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
 }
 
 int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
@@ -636,13 +634,11 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     if (((uintptr_t)x[j] & 15) || ((uintptr_t)y[j] & 7) || (w_base[j] && ((uintptr_t)w_base[j] & 15))) return DZ_EALIGN;
     n_total += N[j];
   }
-  if (n_total > WS_MAX_ROWS) return DZ_ESHAPE;
   if (!workspace || workspace_bytes < dz_workspace_bytes(T, K, (int)n_total)) return DZ_EWORKSPACE;
 
   hipStream_t st = (hipStream_t)stream;
   int* perm = (int*)((char*)workspace + WS_HEADER) + 1024;
-  unsigned* counters = (unsigned*)((char*)workspace + WS_HEADER + WS_PERM_BYTES);
-  char* region = (char*)workspace + WS_HEADER + WS_PERM_BYTES + WS_COUNTER_BYTES;
+  char* region = (char*)workspace + WS_HEADER + WS_PERM_BYTES;
   MdlParams P[DZ_MAX_BATCH_CALLS];
   for (int j = 0; j < ncalls; ++j) {
     size_t cb, mb, sb;
@@ -659,8 +655,6 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     Q.idx = (const long long*)indices;
     Q.y = (_Float16*)y[j];
     Q.status = (unsigned*)workspace;
-    Q.counters = counters;
-    counters += (size_t)(N[j] / DZ_NPAIR) * 4;
     Q.partials = (float*)region;
     region += (size_t)MAX_KSPLIT * 32 * (size_t)N[j] * 4;
     Q.codes_slot_u4 = (long long)(cb / 16);
@@ -679,7 +673,7 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
   // groups to the chunks of 32; one launch carries all chunks
   if (T > 32 && !order)
     hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
-  return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override);
+  return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override.load(std::memory_order_relaxed));
 }
 
 int dz_token_order(const int64_t* indices, int T, int S, int32_t* order, void* stream) {

@@ -7,28 +7,31 @@
 //     with ballots (no sort, no barrier): output columns stay in token order and each delta gets a
 //     per-column mask.  Batches that arrive sorted by id (as the reference's scheduler delivers
 //     them) touch fewer column tiles;
-//   * then everything else is requested at once, in the order it will be used: activations slice
-//     (straight into LDS), the packed words of up to 8 deltas (two batches of 4), the base tile.
-//     The number of requests is fixed, so the wait in front of each use is exact and the deltas
-//     are multiplied while the base tile is still on its way;
+//   * the activations slice goes first (straight into LDS; it does not depend on the ids), then
+//     the packed words of up to 8 deltas (two batches of 4); the base tile is requested once the
+//     first batch has been multiplied, so that a wavefront is not held at its request queue while
+//     data it could work on has arrived.  The number of requests is fixed, so the wait in front
+//     of each use is exact;
 //   * one read of the dense operand (activations, from the wavefront's own LDS slice) feeds every
 //     delta of the current batch (2:4-sparse v_smfmac_f32_16x16x64_f16, unpacked codes as the
 //     sparse operand, stored positions as its index operand); the base tile follows on
 //     v_mfma_f32_16x16x32_f16;
 //   * partial sums of the 4 wavefronts meet in LDS; when K is split over several workgroups the
-//     per-chunk sums go to a workspace and the last workgroup to arrive adds them in a fixed
-//     order (deterministic) and writes y.
+//     per-slice sums go to a workspace whose slots are their own "ready" marks (all zero bits =
+//     empty): the workgroups of all but the last slice store and leave, the workgroup of the last
+//     slice adds the slices in a fixed order (deterministic), writes y and empties the slots.
 #include "../../include/dz_amd.h"
 #include "dz_device.h"
 
 namespace {
 
 constexpr int WK32 = 4;
+constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is about a microsecond)
 
 // The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
 template <int BITS, int TT, bool PRE, bool HAS_BASE>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
-                                           unsigned char* smem, int& s_last) {
+                                           unsigned char* smem) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? 4 : (TT == 2 ? 2 : 3);   // deltas per batch; two batches are in flight
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
@@ -74,14 +77,26 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // one 32-bit lane offset.
   auto issue_x = [&](int kb, int lane_r) {
     const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
+    const int c = lane_r & 31;
+    if (P.perm) {
 #pragma unroll
-    for (int i = 0; i < NX; ++i) {
-      const int t = min(2 * i + (lane_r >> 5), Tc - 1), c = lane_r & 31;
-      const int row = __builtin_amdgcn_ds_bpermute(t << 2, prow);
-      const unsigned off = (unsigned)row * Kb + (unsigned)((c ^ (t & 15)) << 4);
-      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
-                                       (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
-                                       16, 0, 0);
+      for (int i = 0; i < NX; ++i) {
+        const int t = min(2 * i + (lane_r >> 5), Tc - 1);
+        const int row = __builtin_amdgcn_ds_bpermute(t << 2, prow);
+        const unsigned off = (unsigned)row * Kb + (unsigned)((c ^ (t & 15)) << 4);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
+                                         (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
+                                         16, 0, 0);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NX; ++i) {
+        const int t = min(2 * i + (lane_r >> 5), Tc - 1);
+        const unsigned off = (unsigned)(tok0 + t) * Kb + (unsigned)((c ^ (t & 15)) << 4);
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)(xb + off),
+                                         (__attribute__((address_space(3))) void*)(xw + 2 * i * DZ_KBLOCK),
+                                         16, 0, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   };
@@ -128,7 +143,18 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   long long id = -1;
   if (lane < Tc) {
     prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
-    id = P.idx[prow];
+    const long long* ip = P.idx + prow;
+    // requested outside the compiler's bookkeeping: it would wait for the LDS-direct loads that
+    // follow as well (it cannot tell them apart); the wait below counts them instead
+    asm volatile("global_load_dwordx2 %0, %1, off" : "+v"(id) : "v"(ip) : "memory");
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  {
+    // round 0's activations (a wavefront without a k-block fetches a slice it will not use)
+    int lane_0 = lane;
+    asm volatile("" : "+v"(lane_0));
+    issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(id) : "n"(NX) : "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -140,11 +166,12 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     int lane_r = lane;
     asm volatile("" : "+v"(lane_r));
 
+    // the activations do not depend on the ids: they go first, the ids are awaited behind them
+    if (r > 0 && active) issue_x(kb, lane_r);
     if (r == 0) {
-      // nothing is requested before the ids are in (see above)
       if (lane < Tc) {
         key = (id < 0 || id >= P.S) ? 0 : (int)id + 1;
-        if ((id < -1 || id >= P.S) && np == 0 && kc == 0 && wave == 0) atomicOr(P.status, 1u);
+        if ((id < -1 || (P.S > 0 && id >= P.S)) && np == 0 && kc == 0 && wave == 0) atomicOr(P.status, 1u);   // without slots the ids mean nothing
       }
       // tokens that carry a delta; lanes >= T never match
       mdelta = __builtin_amdgcn_ballot_w64(key != 0 && key != 0x7fffffff);
@@ -187,19 +214,16 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
       }
     };
 
-    // ---- issue order: activations (L2 -> LDS), packed deltas of two batches, base tile
-    issue_x(kb, lane_r);
+    // ---- issue order: activations (L2 -> LDS, above), packed deltas of two batches, base tile
     load_batch(ring[0], rsc[0]);
     load_batch(ring[1], rsc[1]);
-    __builtin_amdgcn_sched_barrier(0);
-    if (HAS_BASE) issue_base(kb, lane_r);
     __builtin_amdgcn_sched_barrier(0);
     if (r == 0) DZ_TS(2);
     // Loads return in order and the activations were requested first: once only the loads issued
     // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
     // not order LDS reads after LDS-direct loads by itself.)
     {
-      constexpr int later = 2 * G * (BITS == 2 ? 2 : 3) + (HAS_BASE ? 16 : 0);
+      constexpr int later = 2 * G * (BITS == 2 ? 2 : 3);
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
       // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
       // believes one outstanding, turns every later vmcnt wait into vmcnt(0)
@@ -287,6 +311,9 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // first two batches in straight-line code; their data arrives before the base tile does
     consume(ring[0], rsc[0]);
     if (ld_m) load_batch(ring[0], rsc[0]);
+    __builtin_amdgcn_sched_barrier(0);
+    if (HAS_BASE) issue_base(kb, lane_r);
+    __builtin_amdgcn_sched_barrier(0);
     consume(ring[1], rsc[1]);
     if (ld_m) load_batch(ring[1], rsc[1]);
     // ---- base: dense matrix-core product over all token tiles
@@ -356,8 +383,8 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
       *(h4_t*)yp = o;
     }
   };
-  // partial sums of one k-chunk: [chunk][n-pair][item][4 values][64 lanes] floats.  They are
-  // written and read with agent-scope accesses (write-through / cache-bypassing), so that no
+  // partial sums of one K-slice: [chunk][slice][n-pair][item][4 values][64 lanes] floats.  They
+  // are written and read with agent-scope accesses (write-through / cache-bypassing), so that no
   // whole-cache write-back or invalidate is needed to pass them between XCDs.
   auto part_ptr = [&](int kc2, int item) -> float* {
     return P.partials + (((size_t)(ch * P.nsplit + kc2) * P.NP + np) * (2 * TT) + item) * 256 + lane;
@@ -390,41 +417,60 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     if (has_item) store_item(sum);
     return;
   }
-  if (has_item) {
-    float* pp = part_ptr(kc, wave);
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      __hip_atomic_store(pp + 64 * e, sum[e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the sums have left this CU
-  }
-  __syncthreads();
-  if (tid == 0) {
-    const unsigned old = atomicAdd(P.counters + ch * P.NP + np, 1u);
-    s_last = (old == (unsigned)(P.nsplit - 1));
-  }
-  __syncthreads();
-  DZ_TS(8);
-  if (s_last) {
+  // The partial sums carry their own "ready" mark: a slot of the workspace is all zero bits while
+  // empty, and a sum of +0.0 is written as -0.0.  The workgroups of the K-slices 0 .. nsplit - 2
+  // store theirs and leave at once.  The workgroup of the last K-slice (dispatched after them) reads
+  // the slots until every value is in, adds them in slice order, its own last, writes y and empties
+  // the slots again.  The wait is bounded: if a slot stays empty the launch reports it in the
+  // status word instead of spinning for ever.
+  if (kc != P.nsplit - 1) {
     if (has_item) {
-      // eight K-slices per turn: all their loads are in flight together (one memory round trip
-      // instead of eight), the additions stay in slice order
-      f4_t tot = {0.f, 0.f, 0.f, 0.f};
-      for (int k0 = 0; k0 < P.nsplit; k0 += 8) {
-        f4_t v[8];
+      unsigned* pp = (unsigned*)part_ptr(kc, wave);
+      const u4_t sb = __builtin_bit_cast(u4_t, sum);
+      __hip_atomic_store(pp, sb[0] ? sb[0] : 0x80000000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pp + 64, sb[1] ? sb[1] : 0x80000000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pp + 128, sb[2] ? sb[2] : 0x80000000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pp + 192, sb[3] ? sb[3] : 0x80000000u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    DZ_TS(8);
+    return;
+  }
+  if (has_item) {
+    f4_t tot = {0.f, 0.f, 0.f, 0.f};
+    const int nother = P.nsplit - 1;
+    for (int k0 = 0; k0 < nother; k0 += 8) {
+      unsigned v[8][4];
+      int spins = 0;
+      for (;;) {
+        unsigned all = 0xffffffffu;
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const float* pp = part_ptr(min(k0 + u, P.nsplit - 1), wave);
+          const unsigned* pp = (const unsigned*)part_ptr(min(k0 + u, nother - 1), wave);
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
+          for (int e = 0; e < 4; ++e) {
             v[u][e] = __hip_atomic_load(pp + 64 * e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            all = v[u][e] ? all : 0u;
+          }
         }
-#pragma unroll
-        for (int u = 0; u < 8; ++u)
-          if (k0 + u < P.nsplit) tot += v[u];
+        if (__builtin_amdgcn_ballot_w64(all == 0u) == 0ull) break;
+        if (++spins > DZ_SPIN_LIMIT) {
+          if (lane == 0) atomicOr(P.status, 2u);
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
       }
-      store_item(tot);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (k0 + u < nother) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) tot[e] += __builtin_bit_cast(float, v[u][e]);
+          unsigned* pp = (unsigned*)part_ptr(k0 + u, wave);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) __hip_atomic_store(pp + 64 * e, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    if (tid == 0) P.counters[ch * P.NP + np] = 0u;
+    tot += sum;
+    store_item(tot);
   }
   DZ_TS(9);
 }
@@ -436,12 +482,11 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
 template <int BITS, int TT, bool PRE, bool HAS_BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ int s_last;
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
   const int per = P.nsplit * P.nchunk, rem = q % per;
   const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
   if (np >= P.NP) return;
-  mdl32_body<BITS, TT, PRE, HAS_BASE>(P, np, kc, ch, smem, s_last);
+  mdl32_body<BITS, TT, PRE, HAS_BASE>(P, np, kc, ch, smem);
 }
 
 // Several layer calls that share tokens, K and the slot table (the projections a fused layer
@@ -451,7 +496,6 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 template <int BITS, int TT, bool PRE, bool HAS_BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlBatch B) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-  __shared__ int s_last;
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
   const int per = B.p[0].nsplit * B.p[0].nchunk, rem = q % per;
   const int npg = (q / per) * 8 + xcd, kc = rem / B.p[0].nchunk, ch = rem % B.p[0].nchunk;
@@ -459,7 +503,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlB
   // wavefront-uniform choice among the calls (np_end of unused entries repeats the total)
   const int j = (npg >= B.np_end[0]) + (npg >= B.np_end[1]) + (npg >= B.np_end[2]);
   const int first = j == 0 ? 0 : B.np_end[j - 1];
-  mdl32_body<BITS, TT, PRE, HAS_BASE>(B.p[j], npg - first, kc, ch, smem, s_last);
+  mdl32_body<BITS, TT, PRE, HAS_BASE>(B.p[j], npg - first, kc, ch, smem);
 }
 
 // K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
@@ -497,14 +541,11 @@ int launch32(MdlBatch B, int nprob, bool pre, hipStream_t st, int ksplit_overrid
   }
   const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
-  static bool attr_done[8] = {false, false, false, false, false, false, false, false};
+  static std::atomic<unsigned long long> attr_done[8];
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
     const int which = slot + (nprob == 1 ? 0 : 4);
-    if (!attr_done[which]) {
-      if (hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) return DZ_ELAUNCH;
-      attr_done[which] = true;
-    }
+    if (!dz_lds_limit_once(attr_done[which], f, (int)lds)) return DZ_ELAUNCH;
     if (nprob == 1) hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, B.p[0]);
     else hipLaunchKernelGGL(bkern, dim3(grid), dim3(64 * WK32), lds, st, B);
     return DZ_OK;

@@ -157,9 +157,11 @@ int dz_obs_sweep(float* W, const float* hinv_upper, const float* scale, int N, i
                  int prunem, float* err_workspace, float* loss, void* stream);
 
 /* Bytes of device workspace dz_multi_delta_linear needs for these sizes.  The workspace must be
- * zero-filled once before first use; calls leave it ready for the next call (whatever their
- * sizes: the arrival counters sit in a fixed 1 MiB area, which limits one launch to 2 M output
- * rows in total).  Calls that share a workspace must be ordered on one stream. */
+ * zero-filled once before first use; calls leave it zero-filled for the next call, whatever their
+ * sizes (it carries the partial sums of a K dimension split over workgroups; an empty slot is all
+ * zero bits).  Calls that share a workspace must be ordered on one stream.  Word 0 is a status
+ * word: bit 0 = a delta id outside [-1, S) was met (treated as -1), bit 1 = a partial sum did not
+ * arrive within the kernel's bounded wait (the output of that call is then invalid). */
 size_t dz_workspace_bytes(int T, int K, int N);
 
 /* The layer.  x [T, K] fp16 row-major; w_base [N, K] fp16 row-major or NULL (delta only);
@@ -258,8 +260,9 @@ int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* c
                         int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
                         uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
 
-/* Tuning hook used by the benchmark: override the split of K across workgroups of the fused
- * kernel (0 = automatic). */
+/* Debugging and tuning hook, not part of the layer's interface: overrides, for every later call of
+ * the process, the number of K-slices of the fused kernel (0 = automatic, the default).  The
+ * results do not depend on it beyond the order of the fp32 additions. */
 void dz_set_ksplit(int nsplit);
 
 #ifdef __cplusplus
