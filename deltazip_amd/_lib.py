@@ -37,6 +37,7 @@ SIGNATURES = {
     "dz_workspace_bytes": (_sz, [_i, _i, _i]),
     "dz_multi_delta_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i,
                                    _vp, _sz, _vp]),
+    "dz_multi_delta_linear_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16_pair": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16_grouped": (_i, [_vp, _vp, _vp, C.c_longlong, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp]),

@@ -436,6 +436,28 @@ constexpr size_t WS_HEADER = 256;  // status word
 constexpr int MAX_KSPLIT = 16;
 constexpr size_t WS_PERM_BYTES = 4096 + (size_t)DZ_MAX_TOKENS_FUSED * 4;   // reserved + token order
 
+// Workspace of dz_multi_delta_linear_static: device memory that belongs to the library's code
+// object (zero bits when the object is loaded; every GPU holds its own copy at its own address).
+// Host code must not use the array's name as an address: it asks the runtime for the device
+// address once per device (static_scratch_ptr) and passes that on.
+constexpr size_t STATIC_SCRATCH_BYTES =
+    WS_HEADER + WS_PERM_BYTES + (size_t)MAX_KSPLIT * 32 * (size_t)DZ_STATIC_MAX_N * 4;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratch_ptr[MAX_DEVICES];
+
+// Device address of `scratch` on the current device, looked up on the first call per device.
+void* static_scratch_ptr() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+  g_scratch_ptr[dev].store(p, std::memory_order_release);   // two racing threads store the same address
+  return p;
+}
+
 }  // namespace
 
 extern "C" {
@@ -459,6 +481,7 @@ const char* dz_strerror(int code) {
     case DZ_EWORKSPACE: return "workspace missing or too small";
     case DZ_ELAUNCH: return "HIP launch failed";
     case DZ_EALIGN: return "pointer or leading dimension not aligned";
+    case DZ_ESTATICMAX: return "N exceeds DZ_STATIC_MAX_N, the largest layer the library's built-in workspace serves";
     default: return "unknown error";
   }
 }
@@ -694,6 +717,17 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base, const void*
   return dz_multi_delta_linear_batch(1, &x, &w_base, &codes_stacked, &meta_stacked, &scales_stacked, indices, &y,
                                      &N, &ldy, T, K, S, bits, group_size, accumulate, nullptr, workspace,
                                      workspace_bytes, stream);
+}
+
+int dz_multi_delta_linear_static(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
+                                 const void* meta_stacked, const void* scales_stacked,
+                                 const int64_t* indices, uint16_t* y, int T, int K, int N, int S, int bits,
+                                 int group_size, int accumulate, int ldy, void* stream) {
+  if (N > DZ_STATIC_MAX_N) return DZ_ESTATICMAX;
+  void* ws = static_scratch_ptr();
+  if (!ws) return DZ_ELAUNCH;
+  return dz_multi_delta_linear(x, w_base, codes_stacked, meta_stacked, scales_stacked, indices, y, T, K, N, S,
+                               bits, group_size, accumulate, ldy, ws, STATIC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

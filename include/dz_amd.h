@@ -42,9 +42,11 @@ extern "C" {
 #define DZ_EWORKSPACE   -8   /* workspace missing or too small                             */
 #define DZ_ELAUNCH      -9   /* the HIP runtime refused the launch                         */
 #define DZ_EALIGN      -10   /* pointer not aligned as required                            */
+#define DZ_ESTATICMAX  -11   /* dz_multi_delta_linear_static: N above DZ_STATIC_MAX_N       */
 
 #define DZ_MAX_TOKENS_FUSED 128   /* largest T the fused decode kernel takes in one launch   */
 #define DZ_MAX_BATCH_CALLS 4      /* layer calls dz_multi_delta_linear_batch takes at once    */
+#define DZ_STATIC_MAX_N 16384      /* largest N dz_multi_delta_linear_static takes             */
 #define DZ_MAX_SLOTS_SEGMENT 768   /* largest S dz_segment takes (its tables live in LDS)      */
 #define DZ_MAX_SLOTS_MAP 4096      /* largest S dz_map_ids takes (the slot table lives in LDS) */
 
@@ -181,6 +183,23 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
                           int T, int K, int N, int S, int bits, int group_size,
                           int accumulate, int ldy, void* workspace, size_t workspace_bytes,
                           void* stream);
+
+/* dz_multi_delta_linear for callers that cannot allocate device memory or hand over a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has
+ * no counterpart in the reference.  Same arguments, results and error codes as
+ * dz_multi_delta_linear without the workspace: the partial sums, the token order and the status
+ * word live in a fixed array of device memory inside the library's code object (32 MiB + 5 KiB
+ * per GPU the library runs on, held until the process ends), which serves N <= DZ_STATIC_MAX_N;
+ * a larger N returns DZ_ESTATICMAX.  The call allocates nothing and frees nothing; its first
+ * call on a device looks the array's address up (hipGetSymbolAddress), which is the only set-up.
+ * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
+ * host threads) race; order them on one stream.  The array is all zero bits at load and every
+ * call leaves the partial-sum slots zero again, as with a caller's workspace. */
+int dz_multi_delta_linear_static(const uint16_t* x, const uint16_t* w_base,
+                                 const void* codes_stacked, const void* meta_stacked,
+                                 const void* scales_stacked, const int64_t* indices, uint16_t* y,
+                                 int T, int K, int N, int S, int bits, int group_size,
+                                 int accumulate, int ldy, void* stream);
 
 /* Up to DZ_MAX_BATCH_CALLS layer calls in one launch: calls that share the tokens (T, indices),
  * K, S, bits and group_size -- the projections the reference holds as one fused layer (q/k/v:
