@@ -35,8 +35,24 @@ T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1    # the default workload (configurati
 
 # HBM bytes per launch (average over the 4 launches of a step) of the default workload, from
 # rocprofv3 FETCH_SIZE and WRITE_SIZE runs of this script, each scaled by what the same counter
-# reads for the --calib-copy-mib copy kernel; the figures are in profiles/*__hbm_traffic.txt.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 216410302
+# reads for the --calib-copy-mib copy kernel.  The figure belongs to the kernel sources it was
+# measured on: it is reported only while their fingerprint (kernel_fingerprint) still equals the
+# one recorded here with the profile, and withheld (null) once the kernel has changed.
+MEASURED_TRAFFIC = {
+    "bytes_per_launch": 216410302,
+    "profile": "profiles/dz_mdl32_kernel__llama7b_decode_t32_d8_2bit__hbm_traffic.txt",
+    "kernel_sha256": "to-be-measured",
+}
+KERNEL_SOURCES = ("deltazip_amd/csrc/dz_mdl32.hip", "deltazip_amd/csrc/dz_device.h", "deltazip_amd/csrc/dz_layout.h")
+
+
+def kernel_fingerprint():
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()
 
 
 def algorithmic_bytes(K, N, T, bits, d_present, G=1):
@@ -68,13 +84,39 @@ def parity_check(dev):
             "ok": bool(exact and err <= 1e-2)}
 
 
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline():
     """The reference's CPU path (unpack -> dequant -> W_base + delta in fp32 -> matmul per id) on
-    this host, one call of each distinct layer shape; a step is 4 + 2 + 1 such calls."""
+    this host.  Per distinct layer shape: 3 untimed calls, then the median of 5; a step is
+    4 + 2 + 1 such calls.  Reported: all threads with the dequantisation on every call (what the
+    naive reference does; `value`), all threads with the deltas dequantised beforehand (matmul
+    only, a lower bound), and one thread (smallest shape only, scaled by weight elements)."""
     from oracle import cpu_path
     g = torch.Generator().manual_seed(7)
     ids = torch.sort(torch.randint(0, NUM_DELTAS, (T,), generator=g)).values
-    per_shape, total = {}, 0.0
+    nthreads = torch.get_num_threads()
+
+    def timed(fn, warm, reps):
+        for _ in range(warm):
+            fn()
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    per_shape, per_shape_mm, total, total_mm, one_thread = {}, {}, 0.0, 0.0, None
+    step_elems = sum(K * N for _, K, N in SHAPES)
     for (K, N), count in (((4096, 4096), 4), ((4096, 11008), 2), ((11008, 4096), 1)):
         pf = 32 // BITS
         deltas = []
@@ -85,19 +127,32 @@ def cpu_baseline():
             deltas.append((qw, qz, sc, torch.zeros(K, dtype=torch.int32)))
         wb = (torch.randn((N, K), generator=g) * 0.02).half()
         x = torch.randn((T, K), generator=g).half()
-        reps = []
-        for _ in range(3):                       # first call warms the allocator and BLAS threads
-            t0 = time.perf_counter()
-            cpu_path.forward_cpu(x, wb, deltas, ids, BITS)
-            reps.append(time.perf_counter() - t0)
-        dt = float(np.median(reps[1:]))
-        per_shape[f"{K}x{N}"] = dt
+        dt = timed(lambda: cpu_path.forward_cpu(x, wb, deltas, ids, BITS), 3, 5)
+        pre = [cpu_path.dequant_torch(*d, BITS) for d in deltas]
+        dm = timed(lambda: cpu_path.forward_cpu(x, wb, deltas, ids, BITS, predequantised=pre), 3, 5)
+        per_shape[f"{K}x{N}"], per_shape_mm[f"{K}x{N}"] = dt, dm
         total += count * dt
-    return {"value": T / total, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": "each distinct projection shape (4096x4096, 4096x11008, 11008x4096) called 3 times, "
-                      "median of the last 2; dequant + fp32 add + matmul per delta on every call, as the "
-                      "naive reference does; step time = 4*t1 + 2*t2 + t3",
-            "seconds_per_step": total, "seconds_per_shape": per_shape, "os_cpu_count": os.cpu_count()}
+        total_mm += count * dm
+        if one_thread is None:
+            torch.set_num_threads(1)
+            try:
+                d1 = timed(lambda: cpu_path.forward_cpu(x, wb, deltas, ids, BITS), 1, 3)
+            finally:
+                torch.set_num_threads(nthreads)
+            one_thread = {"threads": 1, "seconds_4096x4096": d1,
+                          "tokens_per_s_extrapolated": T / (d1 * step_elems / (K * N)),
+                          "sample": "4096x4096 only, 1 untimed call + median of 3; step time scaled by weight "
+                                    "elements (x%.2f)" % (step_elems / (K * N))}
+        del deltas, pre
+    return {"value": T / total, "unit": "tokens/s", "cores": nthreads, "kind": "port",
+            "sample": "each distinct projection shape (4096x4096, 4096x11008, 11008x4096): 3 untimed calls, "
+                      "median of 5; dequant + fp32 add + matmul per delta on every call, as the naive "
+                      "reference does; step time = 4*t1 + 2*t2 + t3",
+            "seconds_per_step": total, "seconds_per_shape": per_shape,
+            "matmul_only": {"value": T / total_mm, "unit": "tokens/s", "seconds_per_step": total_mm,
+                            "seconds_per_shape": per_shape_mm,
+                            "what": "deltas dequantised beforehand; fp32 add + matmul per delta (lower bound)"},
+            "one_thread": one_thread, "cpu_model": _cpu_model(), "os_cpu_count": os.cpu_count()}
 
 
 SHAPES_13B = [("q_proj", 5120, 5120), ("k_proj", 5120, 5120), ("v_proj", 5120, 5120), ("o_proj", 5120, 5120),
@@ -269,18 +324,31 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for i in range(warmup):
-        step(i)
+    # Untimed steps: at least --warmup of them, and at least MIN_WARM_SECONDS of back-to-back launches,
+    # so that the clocks have ramped whatever --warmup says (a handful of 0.2 ms steps is over before
+    # the power management has reacted).
+    MIN_WARM_SECONDS = 0.25
+    done, t_w = 0, time.perf_counter()
+    while done < warmup or time.perf_counter() - t_w < MIN_WARM_SECONDS:
+        for _ in range(max(1, min(50, warmup - done))):
+            step(done)
+            done += 1
+        torch.cuda.synchronize()
+    warm_steps_run = done
+    # exactly `steps` timed steps; an event in front of every step (on the stream the kernels are
+    # launched on) gives the per-step times as well
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    e0.record()                                  # on the stream the kernels are launched on
     for i in range(steps):
+        evs[i].record()
         step(i)
-    e1.record()
+    evs[steps].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    gpu_s = e0.elapsed_time(e1) * 1e-3
+    gpu_s = evs[0].elapsed_time(evs[steps]) * 1e-3
+    step_ms = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(steps))
+    median_step_ms = step_ms[steps // 2]
 
     def abytes(K, N):
         return algorithmic_bytes(K, N, T, bits, d_present, 1 if gs == -1 else K // gs)
@@ -312,7 +380,9 @@ def main():
         achieved = (step_bytes / len(groups)) / avg_launch_s / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH if default_workload else None,
+                    "traffic": (MEASURED_TRAFFIC["bytes_per_launch"]
+                                if default_workload and MEASURED_TRAFFIC["kernel_sha256"] == kernel_fingerprint() else None),
+                    "traffic_profile": MEASURED_TRAFFIC["profile"],
                     "kernel": "dz_mdl32_kernel" if all(len(g) == 1 for g in groups) else "dz_mdl32_kernel + dz_mdl32_batch_kernel (same body)",
                     "algorithmic_bytes_per_launch": step_bytes // len(groups),
                     "avg_launch_us": round(avg_launch_s * 1e6, 2)}
@@ -331,6 +401,8 @@ def main():
         "unit": "tokens/s",
         "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step,
+        "ms_per_step_median": round(median_step_ms, 5), "ms_per_step_min": round(step_ms[0], 5),
+        "warmup_steps_run": warm_steps_run,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": cfg["name"] + ("" if args.unsorted or cfg["ids"] in ("zeros", "blocks")

@@ -1,6 +1,7 @@
 """The reference's CPU-runnable forward, restated with torch CPU ops.  TEST INFRASTRUCTURE ONLY.
 
-Used by the benchmark's CPU-baseline leg (and cross-checked against the numpy oracle in tests):
+Used by the benchmark's CPU-baseline leg; tests/test_cpu_path.py holds it to the numpy oracle
+(dequant_torch == dequant_gptq bit for bit, forward_cpu == forward_ref):
   * unpack + dequantise exactly as QuantLinear.forward does
     (serving/vllm/delta/quant_linears/quant_linear_naive.py:39-67): bitwise_right_shift by the
     per-position shifts, mask, zeros + 1, scales[g_idx] * (weight - zeros[g_idx]) in fp16;

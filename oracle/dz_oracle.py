@@ -263,19 +263,6 @@ def forward_token_loop(x16, w_base16, delta_t_list, ids) -> np.ndarray:
     return y
 
 
-def forward_naive_fp16(x16, w_base16, delta_t_list, ids) -> np.ndarray:
-    """The reference's fp16 serving arithmetic (quant_linear_naive.py:80: matmul(x.half(),
-    W) in fp16) added to an fp16 base product.  Reported beside the fp32 result, not gated."""
-    x = torch.from_numpy(np.ascontiguousarray(x16))
-    wb = torch.from_numpy(np.ascontiguousarray(w_base16))
-    y = (x.float() @ wb.float().t()).half()
-    for i, d in enumerate(ids):
-        if d >= 0:
-            dt = torch.from_numpy(np.ascontiguousarray(delta_t_list[int(d)]))
-            y[i] = y[i] + (x[i].float() @ dt.float()).half()
-    return y.numpy()
-
-
 def rel_err(y, y_ref) -> float:
     """max |y - y_ref| / max(|y_ref|, 1e-3 * max|y_ref|): the layer-output parity metric."""
     y = np.asarray(y, dtype=np.float64)
