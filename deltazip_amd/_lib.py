@@ -19,6 +19,7 @@ SIGNATURES = {
     "dz_strerror": (C.c_char_p, [_i]),
     "dz_native_sizes": (_i, [_i, _i, _i, _i, C.POINTER(_sz), C.POINTER(_sz), C.POINTER(_sz)]),
     "dz_repack_2of4": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "dz_unrepack_2of4": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "dz_dequant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "dz_merge": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp]),
     "dz_segment": (_i, [_vp, _i, _i, _vp, _vp, _vp]),

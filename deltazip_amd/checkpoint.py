@@ -35,6 +35,9 @@ from . import ops
 
 CHECKPOINT_NAME = "deltazip-compressed.safetensors"
 CONFIG_NAME = "compress_config.json"
+# safetensors metadata entry that marks a serving-layout file as holding this library's bit layout
+LAYOUT_KEY = "dz_layout"
+NATIVE_LAYOUT = "native-gfx950-v1"
 
 # sub-module -> (fused module, position inside it); llama-style naming, the same table the
 # serving model declares as `packed_modules_mapping` (model_executor/models/llama.py:299-309)
@@ -210,15 +213,27 @@ class DeltaModel:
 
     @classmethod
     def from_tensors(cls, tensors: Dict[str, torch.Tensor], id: int, compress_config: CompressionConfig,
-                     pin_memory: Optional[bool] = None) -> "DeltaModel":
+                     pin_memory: Optional[bool] = None, layout: Optional[str] = None) -> "DeltaModel":
         """From a state dict in either layout: GPTQ-style keys (`*.qzeros` present) are converted
-        first; serving-layout keys (`{module}.0.*`) are taken as they are."""
+        first; serving-layout keys (`{module}.0.qweight/.scales/.meta`) are taken as they are, but only
+        when `layout` says that their bits are this library's (`NATIVE_LAYOUT`).  The reference's own
+        `save_compressed` writes its third-party kernel's (Marlin-style) bit layout under the same
+        file name, key names and shapes (deltazip/modeling/_base.py:636-641,
+        serving/vllm/delta/models.py:236-244): such tensors cannot be told apart by looking at them
+        and would decode to wrong weights, so they are refused."""
         if compress_config.lossless != "none":
             raise NotImplementedError("losslessly packed checkpoints are not supported")
         if compress_config.bits not in (2, 4):
             raise NotImplementedError("Only 2 and 4 bits are supported.")
         if any(k.endswith(".qzeros") for k in tensors):
             tensors = convert_model(tensors, bits=compress_config.bits)
+        elif any(k.endswith(".0.qweight") for k in tensors) and layout != NATIVE_LAYOUT:
+            raise ValueError(
+                "serving-layout tensors ({module}.0.qweight/.scales/.meta) without the layout mark "
+                f"{LAYOUT_KEY}={NATIVE_LAYOUT}: a file written by the reference's save_compressed holds "
+                "Marlin-layout bits under the same names and shapes, which this library cannot read. "
+                "Load the GPTQ-style checkpoint ({module}.qweight/.qzeros/.scales/.g_idx) instead, or pass "
+                f"layout='{NATIVE_LAYOUT}' for tensors that convert_model / compress_model of this library made.")
         pin = torch.cuda.is_available() if pin_memory is None else pin_memory
 
         def host(t: torch.Tensor) -> torch.Tensor:
@@ -239,21 +254,41 @@ class DeltaModel:
 
     @classmethod
     def from_checkpoint(cls, path_or_name: str, id: int, device: Optional[int] = None,
-                        pin_memory: Optional[bool] = None) -> "DeltaModel":
-        """Read `deltazip-compressed.safetensors` + `compress_config.json` from a directory."""
+                        pin_memory: Optional[bool] = None, layout: Optional[str] = None) -> "DeltaModel":
+        """Read `deltazip-compressed.safetensors` + `compress_config.json` from a directory.  The
+        layout of serving-layout tensors is taken from the file's metadata (`save_converted` marks
+        its files) unless `layout` is given."""
         from safetensors import safe_open
         compress_config = CompressionConfig.from_pretrained(path_or_name)
         tensors: Dict[str, torch.Tensor] = {}
         with safe_open(os.path.join(path_or_name, CHECKPOINT_NAME), "pt") as f:
+            if layout is None:
+                layout = (f.metadata() or {}).get(LAYOUT_KEY)
             for key in f.keys():
                 tensors[key] = f.get_tensor(key)
-        return cls.from_tensors(tensors, id, compress_config, pin_memory)
+        return cls.from_tensors(tensors, id, compress_config, pin_memory, layout=layout)
 
 
 def save_converted(tensors: Dict[str, torch.Tensor], compress_config: CompressionConfig, save_dir: str) -> None:
     """Write a serving-layout state dict the way the reference's `save_compressed` does after
-    converting (deltazip/modeling/_base.py:636-645)."""
+    converting (deltazip/modeling/_base.py:636-645), with the metadata entry that tells
+    `from_checkpoint` that the bits are in this library's layout."""
     from safetensors.torch import save_file
+    os.makedirs(save_dir, exist_ok=True)
+    save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(save_dir, CHECKPOINT_NAME),
+              metadata={LAYOUT_KEY: NATIVE_LAYOUT})
+    compress_config.save_pretrained(save_dir)
+
+
+def save_compressed(tensors: Dict[str, torch.Tensor], compress_config: CompressionConfig, save_dir: str) -> None:
+    """Write a GPTQ-style state dict (`compress_model(..., layout="gptq")`) as the reference's
+    `save_compressed` writes an unconverted delta (deltazip/modeling/_base.py:597-648): one
+    `deltazip-compressed.safetensors` with `{module}.qweight/.qzeros/.scales/.g_idx` and the
+    uncompressed parameters, plus `compress_config.json`.  The reference's loaders and this
+    library's `from_checkpoint` both read it."""
+    from safetensors.torch import save_file
+    if any(k.endswith(".0.qweight") for k in tensors):
+        raise ValueError("serving-layout tensors: use save_converted")
     os.makedirs(save_dir, exist_ok=True)
     save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(save_dir, CHECKPOINT_NAME))
     compress_config.save_pretrained(save_dir)
@@ -281,9 +316,14 @@ def _compress_with_hessian(target: torch.Tensor, base: torch.Tensor, inputs: tor
 def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: Dict[str, torch.Tensor],
                    compress_config: CompressionConfig, device="cuda:0",
                    pack_modules: Optional[Dict[str, Tuple[str, int]]] = None,
-                   calibration: Optional[Dict[str, torch.Tensor]] = None) -> Dict[str, torch.Tensor]:
+                   calibration: Optional[Dict[str, torch.Tensor]] = None,
+                   layout: str = "native") -> Dict[str, torch.Tensor]:
     """Fine-tuned model + base model -> serving-layout state dict of the compressed delta (what
-    `convert_model` makes of a checkpoint the reference's compressor wrote), on the GPU.
+    `convert_model` makes of a checkpoint the reference's compressor wrote), on the GPU.  With
+    layout="gptq" the result is the unconverted checkpoint instead, in the reference's own format:
+    `{module}.qweight/.qzeros/.scales/.g_idx` per compressed module (QuantLinear.pack,
+    deltazip/nn_modules/qlinear_cuda.py:144-244; nothing fused) and the remaining parameters under
+    their own names -- what `save_compressed` writes and the reference reads.
 
     Every 2-D `*.weight` outside UNCOMPRESSED_MODULES is compressed as the reference's per-layer
     step does it without calibration data: delta = target.float() - base.float()
@@ -298,6 +338,8 @@ def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: 
         raise NotImplementedError("Only 2 and 4 bits are supported.")
     if not (compress_config.prunen == 2 and compress_config.prunem == 4):
         raise NotImplementedError("only 2:4 pruning (prunen=2, prunem=4) is supported")
+    if layout not in ("native", "gptq"):
+        raise ValueError("layout must be 'native' or 'gptq'")
     pack_modules = PACK_MODULES if pack_modules is None else pack_modules
     bits, gs = compress_config.bits, compress_config.group_size
     out: Dict[str, torch.Tensor] = {}
@@ -314,7 +356,13 @@ def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: 
                 q, m, s = ops.compress_delta(delta.contiguous(), bits, gs)
             native[key[: -len(".weight")]] = (q.cpu(), m.cpu(), s.cpu(), w.shape[1])
         elif key.endswith(".weight") and any(u in key for u in UNCOMPRESSED_MODULES):
-            out[key[: -len(".weight")] + ".0.weight"] = w.detach().cpu()
+            out[key if layout == "gptq" else key[: -len(".weight")] + ".0.weight"] = w.detach().cpu()
+    if layout == "gptq":
+        for module, (q, m, s, K) in native.items():
+            qw, qz, sc, gi = ops.unrepack_native_to_gptq(q, m, s, K, s.shape[-1], bits)
+            out[module + ".qweight"], out[module + ".qzeros"] = qw, qz
+            out[module + ".scales"], out[module + ".g_idx"] = sc, gi
+        return out
     plan: Dict[str, List[Tuple[int, str]]] = {}
     for module, (q, m, s, K) in native.items():
         hit = next((k for k in pack_modules if module.endswith("." + k) or module == k), None)

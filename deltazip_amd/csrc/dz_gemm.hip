@@ -55,6 +55,7 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
     row_lo = P.tiles[tm].row_lo;
     row_hi = P.tiles[tm].row_hi;
     widx = P.tiles[tm].group;
+    if (row_hi <= row_lo) return;   // unused entry of the table
   }
   const int n0 = tn * BN;
   const _Float16* w2 = (P.w2 && widx >= 0) ? P.w2 + (size_t)widx * P.w2_stride : nullptr;

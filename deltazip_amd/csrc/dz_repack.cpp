@@ -95,3 +95,59 @@ extern "C" int dz_repack_2of4(const int32_t* qweight, const int32_t* qzeros, con
       }
   return DZ_OK;
 }
+
+// The inverse: native layout -> the reference's GPTQ-style tensors.  Pruned columns get the
+// zero-point code (they dequantise to 0, as the reference's own packing of a pruned weight does:
+// round(0 / scale) + zero), qzeros holds zero - 1 in every field, g_idx[k] = k / group_size.
+extern "C" int dz_unrepack_2of4(const void* codes_in, const void* meta_in, const uint16_t* scales, int K, int N,
+                                int bits, int group_size, int32_t* out_qweight, int32_t* out_qzeros,
+                                uint16_t* out_scales, int32_t* out_g_idx) {
+  if (!codes_in || !meta_in || !scales || !out_qweight || !out_qzeros || !out_scales) return DZ_EINVAL;
+  size_t cb, mb, sb;
+  int rc = dz_native_sizes(K, N, bits, group_size, &cb, &mb, &sb);
+  if (rc) return rc;
+  const int gs = (group_size == -1) ? K : group_size;
+  const int G = K / gs;
+  const int pf = 32 / bits;
+  const uint32_t mask = (1u << bits) - 1u;
+  const uint32_t zp = 1u << (bits - 1);
+  const int nkb = K / DZ_KBLOCK;
+  const uint32_t* codes = (const uint32_t*)codes_in;
+  const uint32_t* meta = (const uint32_t*)meta_in;
+
+  // every field = zero-point (qweight) and zero-point - 1 (qzeros)
+  uint32_t wz = 0, wq = 0;
+  for (int f = 0; f < pf; ++f) {
+    wz |= zp << (bits * f);
+    wq |= (zp - 1u) << (bits * f);
+  }
+  const size_t nq = (size_t)(K / pf) * N, nz = (size_t)G * (N / pf);
+  for (size_t i = 0; i < nq; ++i) out_qweight[i] = (int32_t)wz;
+  for (size_t i = 0; i < nz; ++i) out_qzeros[i] = (int32_t)wq;
+  memcpy(out_scales, scales, sb);
+  if (out_g_idx)
+    for (int k = 0; k < K; ++k) out_g_idx[k] = k / gs;
+
+  for (int np = 0; np < N / DZ_NPAIR; ++np)
+    for (int kb = 0; kb < nkb; ++kb)
+      for (int la = 0; la < 64; ++la) {
+        const int ga = la >> 4, i = la & 15;
+        for (int j = 0; j < 4; ++j) {
+          const uint32_t mw = meta[dz_meta_word(np, kb, la, j, nkb)];
+          for (int s = 0; s < 2; ++s) {
+            const int n = np * DZ_NPAIR + 16 * s + i;
+            for (int e = 0; e < 8; ++e) {
+              const int pos = (int)((mw >> dz_meta_shift(s, e)) & 3u);
+              const uint32_t c = bits == 2
+                  ? (codes[dz_code2_word(np, kb, la, j, nkb)] >> dz_code2_shift(s, e)) & mask
+                  : (codes[dz_code4_word(np, kb, la, j, s, nkb)] >> dz_code4_shift(e)) & mask;
+              const int k = kb * DZ_KBLOCK + 64 * j + dz_group_k0(ga, e >> 1) + pos;
+              uint32_t& w = (uint32_t&)out_qweight[(size_t)(k / pf) * N + n];
+              const int sh = bits * (k % pf);
+              w = (w & ~(mask << sh)) | (c << sh);
+            }
+          }
+        }
+      }
+  return DZ_OK;
+}

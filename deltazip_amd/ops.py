@@ -79,6 +79,36 @@ def repack_gptq_to_native(qweight: torch.Tensor, qzeros: torch.Tensor, scales: t
     return out_q, out_m, out_s
 
 
+def unrepack_native_to_gptq(qweight: torch.Tensor, meta: torch.Tensor, scales: torch.Tensor, K: int, N: int,
+                            bits: int):
+    """One delta in the native layout -> (qweight, qzeros, scales, g_idx) CPU tensors in the
+    reference's GPTQ-style format (QuantLinear.pack, deltazip/nn_modules/qlinear_cuda.py:144-244):
+    qweight int32 [K*bits/32, N], qzeros int32 [G, N*bits/32], scales fp16 [G, N], g_idx int32 [K].
+    The inverse of `repack_gptq_to_native`; host work."""
+    if bits not in (2, 4):
+        raise NotImplementedError("Only 2 and 4 bits are supported.")
+    qweight = qweight.detach().cpu().contiguous()
+    meta = meta.detach().cpu().contiguous()
+    scales = scales.detach().cpu().contiguous()
+    if scales.dtype != torch.float16 or scales.numel() % N:
+        raise ValueError("scales must be float16 [G, N]")
+    G = scales.numel() // N
+    group_size = -1 if G == 1 else K // G
+    cb, mb, sb = native_sizes(K, N, bits, group_size)
+    if (qweight.numel() * qweight.element_size() != cb or meta.numel() * meta.element_size() != mb
+            or scales.numel() * 2 != sb):
+        raise ValueError("tensors do not match the native layout for these sizes")
+    pf = 32 // bits
+    out_q = torch.empty((K // pf, N), dtype=torch.int32)
+    out_z = torch.empty((G, N // pf), dtype=torch.int32)
+    out_s = torch.empty((G, N), dtype=torch.float16)
+    out_g = torch.empty(K, dtype=torch.int32)
+    rc = _lib.lib().dz_unrepack_2of4(qweight.data_ptr(), meta.data_ptr(), scales.data_ptr(), K, N, bits, group_size,
+                                     out_q.data_ptr(), out_z.data_ptr(), out_s.data_ptr(), out_g.data_ptr())
+    _lib.check(rc, "dz_unrepack_2of4")
+    return out_q, out_z, out_s, out_g
+
+
 def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
@@ -158,8 +188,10 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     """Per-row dense product against the row's own full weight
     (serving/vllm/delta/deltazip_marlin.py:21-53, the lm_head of LogitsProcessorWithDelta):
     out[t] = x[t] @ delta_weights[indices[t]]^T, or x[t] @ base_embedding^T for indices[t] == -1.
-    The rows are grouped by id on the device; like the reference's loop over
-    torch.unique(indices), this reads the group sizes back to the host once."""
+    Where the reference loops over torch.unique(indices) on the host, the rows are grouped by id
+    and cut into row blocks on the device (dz_segment, dz_build_tiles) and two grouped launches
+    multiply them -- the blocks without a delta by the base table, the others by their delta's --
+    so nothing is read back to the host and the call can be captured in a HIP graph."""
     _need_cuda(x, delta_weights, indices, base_embedding)
     if x.dtype != torch.float16 or delta_weights.dtype != torch.float16 or base_embedding.dtype != torch.float16:
         raise ValueError("x and the weights must be float16")
@@ -169,41 +201,24 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
         raise ValueError("shapes: x [T, K], delta_weights [S, N, K], base_embedding [N, K], indices [T]")
     if not (delta_weights.is_contiguous() and base_embedding.is_contiguous()):
         raise ValueError("weights must be contiguous")
+    lib, st = _lib.lib(), _stream()
     perm, seg_off = segment(indices.contiguous(), S)
-    off = seg_off.cpu().tolist()
+    max_tiles = (T + 255) // 256 + min(S + 1, T)
+    tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=x.device)
+    _lib.check(lib.dz_build_tiles(seg_off.data_ptr(), S, tiles.data_ptr(), max_tiles, st), "dz_build_tiles")
+    # two copies of the block table: one keeps the blocks without a delta, one the others (a block
+    # whose row range is empty is skipped by the kernel)
+    with_delta = tiles[:, 2] >= 0
+    base_tiles, delta_tiles = tiles.clone(), tiles.clone()
+    base_tiles[:, 1] = torch.where(with_delta, tiles[:, 0], tiles[:, 1])
+    delta_tiles[:, 1] = torch.where(with_delta, tiles[:, 1], tiles[:, 0])
     perm64 = perm.long()
     xs = x.index_select(0, perm64)
     ys = torch.empty((T, N), dtype=torch.float16, device=x.device)
-    lib, st = _lib.lib(), _stream()
-    weight = lambda d: base_embedding if d < 0 else delta_weights[d]
-    segs = [(off[d + 1], off[d + 2], d) for d in range(-1, S) if off[d + 2] > off[d + 1]]
-    # A group of at most 128 rows is a decode-shaped, HBM-bound product: the fused kernel with no
-    # slots (a dense product with that group's weight) streams the weight once.  Larger groups go
-    # to the matrix-core GEMM, one launch for all of them.
-    small = [g for g in segs if g[1] - g[0] <= MAX_TOKENS_FUSED] if (K % 256 == 0 and N % 32 == 0) else []
-    large = [g for g in segs if g not in small]
-    if small:
-        none_ids = _minus_ones(x.device)
-        ws = _workspace(x.device, MAX_TOKENS_FUSED, K, N)
-        for lo, hi, d in small:
-            rc = lib.dz_multi_delta_linear(xs[lo:hi].data_ptr(), weight(d).data_ptr(), None, None, None,
-                                           none_ids.data_ptr(), ys[lo:hi].data_ptr(), hi - lo, K, N, 0, 2, -1, 0, N,
-                                           ws.data_ptr(), ws.numel(), st)
-            _lib.check(rc, "dz_multi_delta_linear")
-    if large:
-        blocks = lambda lo, hi, g: [(r, min(r + 256, hi), g, 0) for r in range(lo, hi, 256)]
-
-        def launch(w, w2, tiles):
-            tt = torch.tensor(tiles, dtype=torch.int32, device=x.device)
-            _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), w, w2, N * K, tt.data_ptr(), len(tiles), ys.data_ptr(),
-                                               T, K, N, 0, N, st), "dz_gemm_f16_grouped")
-
-        base_tiles = [b for lo, hi, d in large if d < 0 for b in blocks(lo, hi, -1)]
-        delta_tiles = [b for lo, hi, d in large if d >= 0 for b in blocks(lo, hi, d)]
-        if base_tiles:
-            launch(base_embedding.data_ptr(), None, base_tiles)
-        if delta_tiles:
-            launch(None, delta_weights.data_ptr(), delta_tiles)
+    _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), base_embedding.data_ptr(), None, N * K, base_tiles.data_ptr(),
+                                       max_tiles, ys.data_ptr(), T, K, N, 0, N, st), "dz_gemm_f16_grouped")
+    _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), None, delta_weights.data_ptr(), N * K, delta_tiles.data_ptr(),
+                                       max_tiles, ys.data_ptr(), T, K, N, 0, N, st), "dz_gemm_f16_grouped")
     out = torch.empty_like(ys)
     out.index_copy_(0, perm64, ys)
     return out
@@ -581,6 +596,84 @@ def add_delta_slice(y: torch.Tensor, x: torch.Tensor, qweight, qzeros, scales, g
     y2 = y.view(-1, y.shape[-1])[:, y_offset:y_offset + y_slice_size]
     multi_delta_linear(x, None, qweight, scales, meta, indices, bits=bits, out=y2, accumulate=True)
     return y
+
+
+def apply_delta_into(x: torch.Tensor, qweight_stacked: torch.Tensor, qzeros_stacked, scales_stacked: torch.Tensor,
+                     g_idx_stacked, indices: torch.Tensor, output: torch.Tensor, *,
+                     meta_stacked: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Drop-in for the in-place, seven-argument apply_delta of serving/vllm/delta/deltazip.py:78-100:
+    output[i] += x[i] @ dequant(W[indices[i]])^T for all leading dimensions flattened, returned with
+    output's shape.  `meta_stacked` carries the 2:4 positions of the native layout (the reference's
+    add_delta takes them as `meta`, deltazip.py:22); `qzeros_stacked` / `g_idx_stacked` are unused, as
+    in `add_delta`."""
+    x2 = x.view(-1, x.shape[-1])
+    out2 = output.view(-1, output.shape[-1])
+    add_delta(out2, x2, qweight_stacked, qzeros_stacked, scales_stacked, g_idx_stacked, indices.view(-1),
+              meta=meta_stacked)
+    return out2.view_as(output)
+
+
+def apply_delta_packed_nslice(x: torch.Tensor, qweight_stacked: Sequence[torch.Tensor], qzeros_stacked,
+                              scales_stacked: Sequence[torch.Tensor], g_idx_stacked, indices: torch.Tensor,
+                              output: torch.Tensor, output_slices: Sequence[int], *,
+                              meta_stacked: Optional[Sequence[torch.Tensor]] = None,
+                              order: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Drop-in for serving/vllm/delta/deltazip.py:103-153: a layer made of several sublayers packed
+    side by side (q/k/v, gate/up).  For slice j with n_j = output_slices[j] output features,
+    output[:, off_j : off_j + n_j] += x @ dequant(W_j[indices])^T, off_j the sum of the slices before
+    it; index -1 adds nothing.  Up to 128 tokens and 4 slices go in one launch (every slice a call
+    of dz_multi_delta_linear_batch that adds into its columns of `output`); larger batches take one
+    add_delta_slice per slice like the reference.  `meta_stacked[j]`: 2:4 positions of slice j."""
+    n = len(output_slices)
+    if meta_stacked is None:
+        raise ValueError("meta_stacked (2:4 positions of every slice) is required")
+    if not (len(qweight_stacked) >= n and len(scales_stacked) >= n and len(meta_stacked) >= n):
+        raise ValueError("one qweight / scales / meta per output slice is required")
+    K = x.shape[-1]
+    x2 = x.view(-1, K)
+    ind = indices.view(-1)
+    out2 = output.view(-1, output.shape[-1])
+    T = x2.shape[0]
+    if sum(output_slices) > out2.shape[1]:
+        raise ValueError("output_slices exceed the width of output")
+    Ns = [int(v) for v in output_slices]
+    offs = [sum(Ns[:j]) for j in range(n)]
+    fits = (1 <= n <= 4 and T <= MAX_TOKENS_FUSED and out2.dtype == torch.float16 and out2.stride(1) == 1
+            and out2.stride(0) % 4 == 0 and all(o % 4 == 0 for o in offs))
+    if not fits:
+        for j in range(n):
+            add_delta_slice(out2, x2, qweight_stacked[j], None, scales_stacked[j], None, ind, 1.0, offs[j], Ns[j],
+                            meta=meta_stacked[j])
+        return out2.view_as(output)
+    _need_cuda(x2, ind, out2, *qweight_stacked[:n], *scales_stacked[:n], *meta_stacked[:n])
+    if x2.dtype != torch.float16 or not x2.is_contiguous():
+        raise ValueError("x must be contiguous float16")
+    if ind.dtype != torch.int64 or ind.numel() != T or not ind.is_contiguous():
+        raise ValueError("indices must be a contiguous int64 tensor with one entry per token")
+    if out2.shape[0] != T:
+        raise ValueError("output must have one row per token")
+    bits = _bits_from_shapes(qweight_stacked[0], K, Ns[0])
+    S = qweight_stacked[0].shape[0]
+    G = scales_stacked[0][0].numel() // Ns[0]
+    group_size = -1 if G == 1 else K // G
+    for j in range(n):
+        cb, mb, sb = native_sizes(K, Ns[j], bits, group_size)
+        q, m, sc = qweight_stacked[j], meta_stacked[j], scales_stacked[j]
+        if (q.shape[0] != S or q[0].numel() * q.element_size() != cb or m[0].numel() * m.element_size() != mb
+                or sc[0].numel() * sc.element_size() != sb or sc.dtype != torch.float16
+                or not (q.is_contiguous() and m.is_contiguous() and sc.is_contiguous())):
+            raise ValueError("stacked delta tensors do not match the native layout for these sizes")
+    vp = C.c_void_p * n
+    esz = out2.element_size()
+    ws = _workspace(x2.device, T, K, sum(Ns))
+    rc = _lib.lib().dz_multi_delta_linear_batch(
+        n, vp(*[x2.data_ptr()] * n), vp(*[None] * n), vp(*[qweight_stacked[j].data_ptr() for j in range(n)]),
+        vp(*[meta_stacked[j].data_ptr() for j in range(n)]), vp(*[scales_stacked[j].data_ptr() for j in range(n)]),
+        ind.data_ptr(), vp(*[out2.data_ptr() + offs[j] * esz for j in range(n)]), (C.c_int * n)(*Ns),
+        (C.c_int * n)(*[out2.stride(0)] * n), T, K, S, bits, group_size, 1, _order_ptr(order, T, ind.device),
+        ws.data_ptr(), ws.numel(), _stream())
+    _lib.check(rc, "dz_multi_delta_linear_batch")
+    return out2.view_as(output)
 
 
 def set_ksplit(nsplit: int) -> None:

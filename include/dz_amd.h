@@ -71,6 +71,17 @@ int dz_repack_2of4(const int32_t* qweight, const int32_t* qzeros, const uint16_t
                    const int32_t* g_idx, int K, int N, int bits, int group_size,
                    void* out_codes, void* out_meta, void* out_scales);
 
+/* HOST function, host pointers.  The inverse of dz_repack_2of4: one delta in the native layout ->
+ * the reference's GPTQ-style tensors as QuantLinear.pack writes them
+ * (deltazip/nn_modules/qlinear_cuda.py:144-244): qweight [K*bits/32, N] int32 (pruned columns carry
+ * the zero-point code, which dequantises to 0), qzeros [G, N*bits/32] int32 holding zero-1 =
+ * 2^(bits-1)-1 in every field, scales [G, N] fp16, g_idx [K] int32 = k / group_size (may be NULL).
+ * With it a delta compressed here can be saved in the format the reference's save_compressed
+ * writes and its loaders read (deltazip/modeling/_base.py:597-648). */
+int dz_unrepack_2of4(const void* codes, const void* meta, const uint16_t* scales, int K, int N,
+                     int bits, int group_size, int32_t* out_qweight, int32_t* out_qzeros,
+                     uint16_t* out_scales, int32_t* out_g_idx);
+
 /* Dequantise one native delta to fp16, out[n * K + k] (row-major [N, K]).  Bit-exact with
  * QuantLinear.unpack (deltazip/nn_modules/qlinear_cuda.py:246-329): half(float(scale)*(q-zero)). */
 int dz_dequant(const void* codes, const void* meta, const void* scales,

@@ -127,6 +127,26 @@ def test_delta_model_from_checkpoint(dzlib, tmp_path, converted_on_disk):
     assert dm.get_delta("nope") is None
 
 
+def test_serving_layout_tensors_without_the_layout_mark_are_refused(dzlib, tmp_path):
+    """`{module}.0.qweight/.scales/.meta` written by the reference's own save_compressed hold another
+    kernel's bit layout under the same names and shapes; without this library's mark they are not read."""
+    from safetensors.torch import save_file
+    bits = 4
+    sd, _ = make_state_dict(bits, -1, layers=1)
+    cfg = ck.CompressionConfig(bits=bits, sparsity=0.5, prunen=2, prunem=4)
+    conv = ck.convert_model(sd, bits=bits)
+    with pytest.raises(ValueError, match="Marlin"):
+        ck.DeltaModel.from_tensors(conv, 1, cfg, pin_memory=False)
+    assert ck.DeltaModel.from_tensors(conv, 1, cfg, pin_memory=False, layout=ck.NATIVE_LAYOUT).deltas
+    save_file({k: v.contiguous() for k, v in conv.items()}, os.path.join(tmp_path, ck.CHECKPOINT_NAME))   # no mark
+    cfg.save_pretrained(str(tmp_path))
+    with pytest.raises(ValueError, match="Marlin"):
+        ck.DeltaModel.from_checkpoint(str(tmp_path), id=1, pin_memory=False)
+    assert ck.DeltaModel.from_checkpoint(str(tmp_path), id=1, pin_memory=False, layout=ck.NATIVE_LAYOUT).deltas
+    ck.save_converted(conv, cfg, str(tmp_path))                                                          # marked
+    assert ck.DeltaModel.from_checkpoint(str(tmp_path), id=1, pin_memory=False).deltas
+
+
 def test_unsupported_checkpoints_are_refused(dzlib):
     sd, _ = make_state_dict(4, -1, layers=1)
     with pytest.raises(NotImplementedError):
@@ -178,10 +198,50 @@ def test_compress_model_on_gpu(dev, bits, gs):
         assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(ref).view(np.uint16)), tname
     assert torch.equal(out["model.embed_tokens.0.weight"], target["model.embed_tokens.weight"])
     assert torch.equal(out["model.layers.0.input_layernorm.0.weight"], target["model.layers.0.input_layernorm.weight"])
-    dm = ck.DeltaModel.from_tensors(out, 3, cfg, pin_memory=False)
+    dm = ck.DeltaModel.from_tensors(out, 3, cfg, pin_memory=False, layout=ck.NATIVE_LAYOUT)
     assert dm.get_delta("model.layers.0.self_attn.qkv_proj")._compressed and not dm.get_delta("lm_head")._compressed
     with pytest.raises(NotImplementedError):
         ck.compress_model(base, target, ck.CompressionConfig(bits=4, prunen=0, prunem=0), device=dev)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bits,gs", [(4, -1), (2, 128)])
+def test_compress_model_writes_the_reference_format(dev, tmp_path, bits, gs):
+    """compress_model(layout="gptq") + save_compressed: the file holds, per module, byte for byte the
+    qweight/qzeros/scales/g_idx that the reference's pipeline (oracle: compress_delta +
+    pack_codes_gptq) gives for that delta, and loads back to the same serving-layout tensors as
+    the native path."""
+    from safetensors import safe_open
+    g = torch.Generator().manual_seed(13)
+    base, target = {}, {}
+    for name, (n, k) in SHAPES.items():
+        key = f"model.layers.0.{name}.weight"
+        base[key] = (torch.randn(n, k, generator=g) * 0.02).half()
+        target[key] = (base[key].float() + torch.randn(n, k, generator=g) * 1e-3).half()
+    for key, shape in (("model.embed_tokens.weight", (V, H)), ("lm_head.weight", (V, H)), ("model.norm.weight", (H,))):
+        base[key] = torch.randn(*shape, generator=g).half()
+        target[key] = torch.randn(*shape, generator=g).half()
+    cfg = ck.CompressionConfig(bits=bits, group_size=gs, sparsity=0.5, prunen=2, prunem=4)
+    out = ck.compress_model(base, target, cfg, device=dev, layout="gptq")
+    ck.save_compressed(out, cfg, str(tmp_path))
+    with safe_open(os.path.join(tmp_path, ck.CHECKPOINT_NAME), "pt") as f:
+        disk = {k: f.get_tensor(k) for k in f.keys()}
+    for name, (n, k) in SHAPES.items():
+        key = f"model.layers.0.{name}"
+        d32 = target[key + ".weight"].float().numpy() - base[key + ".weight"].float().numpy()
+        codes, scales16, zeros, _ = o.compress_delta(d32, bits, gs)
+        qw, qz, sc, gi = o.pack_codes_gptq(codes, zeros, scales16, bits)
+        assert np.array_equal(disk[key + ".qweight"].numpy(), qw), name
+        assert np.array_equal(disk[key + ".qzeros"].numpy(), qz), name
+        assert np.array_equal(disk[key + ".scales"].numpy().view(np.uint16), sc.view(np.uint16)), name
+        assert np.array_equal(disk[key + ".g_idx"].numpy(), gi.astype(np.int32)), name
+    assert torch.equal(disk["lm_head.weight"], target["lm_head.weight"])
+    dm = ck.DeltaModel.from_checkpoint(str(tmp_path), id=5, pin_memory=False)
+    nat = ck.compress_model(base, target, cfg, device=dev)
+    for mod in ("model.layers.0.self_attn.qkv_proj", "model.layers.0.mlp.gate_up_proj", "model.layers.0.mlp.down_proj"):
+        d = dm.get_delta(mod)
+        assert torch.equal(d.qweight, nat[mod + ".0.qweight"]) and torch.equal(d.meta, nat[mod + ".0.meta"])
+        assert torch.equal(d.scales, nat[mod + ".0.scales"])
 
 
 @pytest.mark.gpu

@@ -168,6 +168,56 @@ def test_add_delta_slices_qkv_and_gate_up(dev):
     assert o.rel_err(yy.cpu().numpy(), o.forward_ref(x_np, None, p["dts"], ids_np)) <= TOL
 
 
+@pytest.mark.parametrize("t,bits,gs", [(20, 4, -1), (100, 2, -1), (7, 4, 128), (300, 2, -1)])
+def test_apply_delta_packed_nslice_and_in_place_apply_delta(dev, t, bits, gs):
+    """The packed-sublayer op and the in-place apply_delta of the reference's non-fused module
+    (deltazip.py:78-153), through its own names: every slice of `output` gains x @ delta_j^T of the
+    token's delta, a base-only token (-1) gains nothing, columns outside the slices stay as they were."""
+    from deltazip_amd import deltazip as dzmod
+    k = 512
+    slices = (128, 64, 96)
+    nd = 4
+    mixed = np.random.default_rng(t).integers(-1, nd, t).astype(np.int64)
+    mixed[:2] = (-1, nd - 1)
+    probs = [make_problem(n, k, bits, gs, nd, t, mixed, 700 + i, dev) for i, n in enumerate(slices)]
+    ids_np = probs[0]["ids_np"]; ids = probs[0]["ids"]; x = probs[0]["x"]; x_np = probs[0]["x_np"]
+    width = sum(slices) + 32                       # 32 columns that belong to no slice
+    lead = (2, t // 2) if t % 2 == 0 else (t,)     # leading dimensions are flattened by the ops
+    y0 = (torch.randn(*lead, width, device=dev) * 0.05).half()
+    y = y0.clone()
+    xin = x.view(*y.shape[:-1], k)
+    got = dzmod.apply_delta_packed_nslice(xin, [p["q"] for p in probs], [None] * 3, [p["s"] for p in probs],
+                                          [None] * 3, ids.view(*y.shape[:-1]), y, slices,
+                                          meta_stacked=[p["m"] for p in probs])
+    torch.cuda.synchronize()
+    assert got.shape == y.shape and got.data_ptr() == y.data_ptr()
+    y2, y02 = y.view(-1, width), y0.view(-1, width)
+    off = 0
+    for p, n in zip(probs, slices):
+        ref = y02[:, off:off + n].float().cpu().numpy() + o.forward_ref(x_np, None, p["dts"], ids_np)
+        assert o.rel_err(y2[:, off:off + n].cpu().numpy(), ref) <= TOL
+        base_rows = torch.from_numpy(ids_np < 0).to(dev)
+        assert torch.equal(y2[base_rows, off:off + n], y02[base_rows, off:off + n])
+        off += n
+    assert torch.equal(y2[:, off:], y02[:, off:])
+    # the same slices one by one give the same bits (one launch or three)
+    y3 = y0.clone().view(-1, width)
+    off = 0
+    for p, n in zip(probs, slices):
+        ops.add_delta_slice(y3, x, p["q"], None, p["s"], None, ids, 1.0, off, n, meta=p["m"])
+        off += n
+    assert torch.equal(y3, y2)
+    # in-place apply_delta over the first slice's delta
+    p = probs[0]
+    z0 = (torch.randn(*y.shape[:-1], slices[0], device=dev) * 0.05).half()
+    z = z0.clone()
+    out = dzmod.apply_delta(xin, p["q"], None, p["s"], None, ids.view(*y.shape[:-1]), z, meta_stacked=p["m"])
+    torch.cuda.synchronize()
+    assert out.shape == z.shape and out.data_ptr() == z.data_ptr()
+    ref = z0.view(-1, slices[0]).float().cpu().numpy() + o.forward_ref(x_np, None, p["dts"], ids_np)
+    assert o.rel_err(z.view(-1, slices[0]).cpu().numpy(), ref) <= TOL
+
+
 def test_deterministic_and_order_independent(dev):
     p = make_problem(128, 1024, 2, -1, 5, 32, "uniform", 55, dev)
     y1 = run_layer(p); y2 = run_layer(p)

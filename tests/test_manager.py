@@ -299,6 +299,41 @@ def test_uncompressed_projection_matches_loop(dev, T, S, N, K):
 
 
 @pytest.mark.gpu
+def test_uncompressed_projection_never_reads_back_to_the_host(dev):
+    """The per-delta output projection is captured into a HIP graph -- which any read-back of the
+    group sizes to the host would refuse -- and every replay, with eager work and synchronisations
+    in between and the ids rewritten in place, gives what the eager call gives."""
+    from deltazip_amd import ops
+    T, S, N, K = 48, 5, 1000, 512
+    rng = np.random.default_rng(99)
+    base_np = (rng.standard_normal((N, K)) * 0.05).astype(np.float16)
+    stack_np = (rng.standard_normal((S, N, K)) * 0.05).astype(np.float16)
+    x_np = rng.standard_normal((T, K)).astype(np.float16)
+    base, stack, x = (torch.from_numpy(a).to(dev) for a in (base_np, stack_np, x_np))
+    ids = torch.from_numpy(rng.integers(-1, S, size=T)).to(dev)
+    ops.apply_delta_uncompressed(x, stack, ids, base)          # first call outside the capture (one-time set-up)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            out = ops.apply_delta_uncompressed(x, stack, ids, base)
+    torch.cuda.current_stream().wait_stream(side)
+    for rep in range(3):
+        new_ids = rng.integers(-1, S, size=T)
+        if rep == 1:
+            new_ids[:] = -1                                     # a batch without any delta
+        ids.copy_(torch.from_numpy(new_ids).to(dev))
+        eager = ops.apply_delta_uncompressed(x, stack, ids, base)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        assert o.rel_err(out.float().cpu().numpy(), o.linear_select_ref(x_np, stack_np, new_ids, base_np)) <= 1e-2
+
+
+@pytest.mark.gpu
 def test_checkpoint_to_manager_to_forward(dev):
     bits = 4
     model = ToyModel(dev)

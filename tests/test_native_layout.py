@@ -84,3 +84,56 @@ def test_repacker_rejects_bad_input(dzlib):
         ops.native_sizes(4096, 4096, 4, 100)          # group size
     with pytest.raises(NotImplementedError):
         ops.native_sizes(4096, 4096, 8)
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+@pytest.mark.parametrize("gs", [-1, 128])
+def test_gptq_writer_is_the_inverse_of_the_repacker(dzlib, bits, gs):
+    """dz_unrepack_2of4 (native -> the reference's qweight/qzeros/scales/g_idx) gives back, byte for
+    byte, the GPTQ tensors the native delta was made from (those are what QuantLinear.pack writes for
+    a 2:4 delta: pruned columns carry the zero-point code), and repacking them gives the same native
+    bytes again."""
+    n, k = 96, 768
+    d = o.make_delta(n, k, 1e-3, bits, gs, 33)
+    q, m, s = ops.repack_gptq_to_native(torch.from_numpy(d["qweight"]), torch.from_numpy(d["qzeros"]),
+                                        torch.from_numpy(d["scales"]), torch.from_numpy(d["g_idx"]), bits)
+    qw, qz, sc, gi = ops.unrepack_native_to_gptq(q, m, s, k, n, bits)
+    assert qw.dtype == torch.int32 and tuple(qw.shape) == d["qweight"].shape
+    assert np.array_equal(qw.numpy(), d["qweight"])
+    assert np.array_equal(qz.numpy(), d["qzeros"])
+    assert np.array_equal(sc.numpy().view(np.uint16), d["scales"].view(np.uint16))
+    assert np.array_equal(gi.numpy(), d["g_idx"].astype(np.int32))
+    q2, m2, s2 = ops.repack_gptq_to_native(qw, qz, sc, gi, bits)
+    assert torch.equal(q2, q) and torch.equal(m2, m) and torch.equal(s2, s)
+    # known fields: qzeros holds zero - 1 = 2^(bits-1) - 1 in every field of every word
+    field = 2 ** (bits - 1) - 1
+    word = sum(field << (bits * f) for f in range(32 // bits))
+    assert (qz.numpy().view(np.uint32) == word).all()
+    # the written tensors dequantise, the reference's way, to the native dequantisation
+    ref = o.dequant_gptq(qw.numpy(), qz.numpy(), sc.numpy(), gi.numpy(), bits)
+    qn = q.numpy().view(np.uint32)
+    codes = qn.reshape(n // 32, k // 256, 64, 4) if bits == 2 else qn.reshape(n // 32, k // 256, 2, 64, 4)
+    nat = o.dequant_native(codes, m.numpy().view(np.uint32).reshape(n // 32, k // 256, 64, 4), s.numpy(), k, n, bits)
+    assert np.array_equal(nat.view(np.uint16), np.ascontiguousarray(ref.T).view(np.uint16))
+
+
+def test_gptq_writer_of_an_all_pruned_delta(dzlib):
+    """Nothing kept anywhere: every qweight word is the zero-point pattern (0x88888888 at 4 bits)."""
+    bits, n, k = 4, 32, 256
+    codes = np.full((k, n), 8, dtype=np.uint8)
+    qw0, qz0, sc0, gi0 = o.pack_codes_gptq(codes, np.full((1, n), 8), np.full((1, n), 0.25, np.float16), bits)
+    q, m, s = ops.repack_gptq_to_native(*(torch.from_numpy(np.ascontiguousarray(v)) for v in (qw0, qz0, sc0, gi0)), bits)
+    qw, qz, sc, gi = ops.unrepack_native_to_gptq(q, m, s, k, n, bits)
+    assert (qw.numpy().view(np.uint32) == 0x88888888).all() and (qz.numpy().view(np.uint32) == 0x77777777).all()
+
+
+def test_gptq_writer_argument_checks(dzlib):
+    one = C.c_void_p(0x1000)
+    f = dzlib.dz_unrepack_2of4
+    assert f(None, one, one, 256, 32, 4, -1, one, one, one, one) == -1
+    assert f(one, one, one, 256, 32, 3, -1, one, one, one, one) == -3
+    assert f(one, one, one, 200, 32, 4, -1, one, one, one, one) == -2
+    assert f(one, one, one, 256, 32, 4, 100, one, one, one, one) == -4
+    with pytest.raises(ValueError):
+        ops.unrepack_native_to_gptq(torch.zeros(10, dtype=torch.int32), torch.zeros(10, dtype=torch.int16),
+                                    torch.zeros((1, 32), dtype=torch.float16), 256, 32, 4)
