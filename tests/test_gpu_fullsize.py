@@ -22,15 +22,29 @@ TOL = 1e-2   # max relative error of fp16 outputs against the fp32 reference (fl
 
 # K, N, bits, group_size, slots, tokens, ids
 CASES = [
+    # configuration 1: one token, one 4-bit delta
     pytest.param(4096, 4096, 4, -1, 1, 1, "single", id="cfg1-7b-4096x4096-4bit-T1"),
+    # configuration 2 (the headline): Llama-2-7B projections, 32 tokens, 8 deltas of 2 bits
     pytest.param(4096, 4096, 2, -1, 8, 32, "uniform", id="cfg2-7b-4096x4096-2bit-T32-D8"),
     pytest.param(4096, 11008, 2, -1, 8, 32, "uniform", id="cfg2-7b-4096x11008"),
     pytest.param(11008, 4096, 2, -1, 8, 32, "uniform", id="cfg2-7b-11008x4096"),
     pytest.param(4096, 12288, 2, -1, 8, 32, "uniform", id="cfg2-7b-fused-qkv"),
-    pytest.param(4096, 4096, 4, 128, 32, 64, "zipf", id="cfg3-7b-4bit-g128-T64-D32-zipf"),
-    pytest.param(5120, 5120, 2, -1, 64, 128, "uniform", id="cfg5-13b-5120x5120-T128-D64"),
+    # configuration 3: the same three shapes, 64 tokens, 32 deltas of 4 bits with group size 128, Zipf ids
+    pytest.param(4096, 4096, 4, 128, 32, 64, "zipf", id="cfg3-7b-4096x4096-4bit-g128-T64-D32-zipf"),
+    pytest.param(4096, 11008, 4, 128, 32, 64, "zipf", id="cfg3-7b-4096x11008-4bit-g128-T64-D32-zipf"),
+    pytest.param(11008, 4096, 4, 128, 32, 64, "zipf", id="cfg3-7b-11008x4096-4bit-g128-T64-D32-zipf"),
+    # configuration 4: Llama-2-13B prefill, 16 requests of 512 tokens, one 2-bit delta each
+    pytest.param(5120, 5120, 2, -1, 16, 8192, "blocks", id="cfg4-13b-5120x5120-prefill-T8192-D16"),
+    pytest.param(5120, 13824, 2, -1, 16, 8192, "blocks", id="cfg4-13b-5120x13824-prefill-T8192-D16"),
+    pytest.param(13824, 5120, 2, -1, 16, 8192, "blocks", id="cfg4-13b-13824x5120-prefill-T8192-D16"),
+    # configuration 5: Llama-2-7B projections at 128 tokens with 64 resident 2-bit deltas (the whole
+    # decode step of that configuration is tests/test_llama_step.py)
+    pytest.param(4096, 4096, 2, -1, 64, 128, "uniform", id="cfg5-7b-4096x4096-T128-D64"),
+    pytest.param(4096, 11008, 2, -1, 64, 128, "uniform", id="cfg5-7b-4096x11008-T128-D64"),
+    pytest.param(11008, 4096, 2, -1, 64, 128, "uniform", id="cfg5-7b-11008x4096-T128-D64"),
+    # further shapes outside the configurations: 13B layers at decode sizes
+    pytest.param(5120, 5120, 2, -1, 64, 128, "uniform", id="13b-5120x5120-T128-D64"),
     pytest.param(13824, 5120, 4, -1, 4, 16, "uniform", id="13b-down-4bit-T16"),
-    pytest.param(5120, 5120, 2, -1, 16, 8192, "blocks", id="cfg4-13b-prefill-T8192-D16"),
 ]
 
 
