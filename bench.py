@@ -174,8 +174,12 @@ CONFIGS = {
     4: dict(name="Llama-2-13B prefill projections, 16 requests x 512 tokens, each bound to its own delta "
                  "(2-bit, 2:4, per-channel)", shapes=SHAPES_13B, T=8192, S=16, bits=2, gs=-1, ids="blocks",
             bound="mfma"),
-    5: dict(name="Llama-2-7B decode projections, 128 tokens, 64 resident deltas (2-bit, 2:4, per-channel), "
-                 "ids uniform", shapes=SHAPES, T=128, S=64, bits=2, gs=-1, ids="uniform", bound="hbm"),
+    5: dict(name="one full decode step of a random-init 32-layer Llama-2-7B (hidden 4096, 32 heads, FFN 11008, "
+                 "fp16): every projection (fused q/k/v, o, fused gate/up, down) is a multi-delta layer created by "
+                 "the delta manager; RMSNorm, rotary and attention over a 1024-token KV context are plain "
+                 "PyTorch-ROCm ops; embedding and output projection on the base tables; 128 decode tokens, "
+                 "64 resident deltas (2-bit, 2:4 sparse, per-channel scales), ids uniform over the deltas",
+            shapes=SHAPES, T=128, S=64, bits=2, gs=-1, ids="uniform", bound="hbm"),
 }
 
 
@@ -192,13 +196,102 @@ def make_ids(kind, t, s, dev, gen, sort):
     return torch.sort(ids).values if sort else ids   # the serving scheduler delivers batches sorted by delta id
 
 
+def timed_steps(step, steps, warmup, min_warm_seconds=0.25):
+    """At least `warmup` untimed steps and at least `min_warm_seconds` of them (so that the clocks
+    have ramped whatever --warmup says), then exactly `steps` timed ones with an event in front of
+    each on the current stream.  Returns (wall seconds, event seconds, sorted per-step ms, warm steps run)."""
+    done, t_w = 0, time.perf_counter()
+    while done < warmup or time.perf_counter() - t_w < min_warm_seconds:
+        for _ in range(max(1, min(50, warmup - done))):
+            step(done)
+            done += 1
+        torch.cuda.synchronize()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        evs[i].record()
+        step(i)
+    evs[steps].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return (wall, evs[0].elapsed_time(evs[steps]) * 1e-3,
+            sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(steps)), done)
+
+
+def run_full_step(args, parity):
+    """Configuration 5: the whole decode step (deltazip_amd/llama_step.py) with every projection a
+    multi-delta layer; reports the step, the share of the projections in it and their HBM fraction."""
+    from deltazip_amd import DeltaConfig, DeltaMapping, create_delta_manager
+    from deltazip_amd.llama_step import LlamaForDecodeStep, LlamaStepConfig
+    from deltazip_amd.synthetic import random_native_stack
+    cfg = CONFIGS[5]
+    T, S, bits, gs, ctx = cfg["T"], cfg["S"], cfg["bits"], cfg["gs"], 1024
+    steps, warmup = args.steps or 10, args.warmup or 2
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(1234)
+    mcfg = LlamaStepConfig(num_hidden_layers=args.layers or 32)
+    model = LlamaForDecodeStep(mcfg, device=dev, generator=gen)
+    mgr = create_delta_manager(model, max_num_seqs=T, max_num_batched_tokens=T, vocab_size=mcfg.vocab_size,
+                               delta_config=DeltaConfig(max_deltas=S, max_bitwidth=bits, group_size=gs))
+    # synthetic deltas written straight into the layers' slot stacks (compressing 64 x 32 real deltas
+    # would take hours); the manager is told that delta d + 1 lives in slot d
+    for name, layer in mgr.modules.items():
+        N, K = layer.base_layer.weight.shape
+        layer.qweight_stacked, layer.meta_stacked, layer.scales_stacked = random_native_stack(K, N, bits, gs, S, dev, gen)
+        layer.bitwidth = [bits] * S
+    mgr.delta_index_to_id = list(range(1, S + 1))
+    ids = torch.sort(torch.randint(1, S + 1, (T,), device=dev, generator=gen)).values.tolist()
+    mgr.set_delta_mapping(DeltaMapping(tuple(ids), tuple(ids)))
+    d_present = len(set(ids))
+    tokens = torch.randint(0, mcfg.vocab_size, (T,), device=dev, generator=gen)
+    kv = model.make_kv_cache(T, ctx, dev)
+    torch.cuda.synchronize()
+
+    wall, gpu_s, step_ms, warm_run = timed_steps(lambda i: model.decode_step(tokens, kv, ctx), steps, warmup)
+    ms_per_step = wall / steps * 1e3
+
+    # the projections alone: the same 4 x layers calls on inputs of the right shape
+    projs = [m for _, m in model.projections()]
+    xs = {K: torch.randn((T, K), device=dev, dtype=torch.float16, generator=gen)
+          for K in {m.base_layer.weight.shape[1] for m in projs}}
+
+    def linears(i):
+        for m in projs:
+            m(xs[m.base_layer.weight.shape[1]])
+    lwall, lgpu, _, _ = timed_steps(linears, steps, warmup)
+    lin_ms = lgpu / steps * 1e3
+    lin_bytes = sum(algorithmic_bytes(m.base_layer.weight.shape[1], m.base_layer.weight.shape[0], T, bits, d_present)
+                    for m in projs)
+    achieved = lin_bytes / (lin_ms * 1e-3) / 1e9
+    out = {
+        "metric": "multi-delta linear tokens/s + achieved HBM TB/s (% peak), Llama-7B shapes",
+        "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": ms_per_step, "ms_per_step_median": round(step_ms[steps // 2], 4), "warmup_steps_run": warm_run,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": cfg["name"] + ", batch sorted by delta id", "baseline_config": 5, "tokens": T,
+                   "deltas": S, "deltas_present": d_present, "bits": bits, "group_size": gs, "kv_context": ctx,
+                   "layers": mcfg.num_hidden_layers, "launches_per_step": len(projs)},
+        "linear_layers": {"ms_per_step": round(lin_ms, 4), "share_of_step": round(lin_ms / (gpu_s / steps * 1e3), 4),
+                          "calls": len(projs), "us_per_call": round(lin_ms * 1e3 / len(projs), 2)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "dz_mdl32_kernel (the projections of the step, timed on their own)",
+                     "algorithmic_bytes_per_launch": lin_bytes // len(projs),
+                     "avg_launch_us": round(lin_ms * 1e3 / len(projs), 2)},
+        "parity": parity,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed steps (default 200; 10 for --config 4)")
     ap.add_argument("--warmup", type=int, default=0, help="untimed steps (default 20; 2 for --config 4)")
     ap.add_argument("--config", type=int, default=2, choices=sorted(CONFIGS), help="BASELINE.json configuration")
-    ap.add_argument("--layers", type=int, default=0, help="distinct decoder layers kept in HBM and visited in turn")
+    ap.add_argument("--layers", type=int, default=0, help="distinct decoder layers kept in HBM and visited in turn "
+                                                       "(--config 5: decoder layers of the model, default 32)")
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ksplit", type=int, default=0)
@@ -221,13 +314,15 @@ def main():
     shapes, T, S, bits, gs = cfg["shapes"], cfg["T"], cfg["S"], cfg["bits"], cfg["gs"]
     steps = args.steps or (10 if args.config == 4 else 200)
     warmup = args.warmup or (2 if args.config == 4 else 20)
-    nlayers = args.layers or {1: 16, 2: 4, 3: 2, 4: 1, 5: 2}[args.config]
+    nlayers = args.layers or {1: 16, 2: 4, 3: 2, 4: 1, 5: 32}[args.config]
     lib = _lib.lib()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(1234)
 
     parity = parity_check(dev)
+    if args.config == 5:
+        return run_full_step(args, parity)
 
     # ---- resident inputs
     ids = make_ids(cfg["ids"], T, S, dev, gen, not args.unsorted)
@@ -324,30 +419,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    # Untimed steps: at least --warmup of them, and at least MIN_WARM_SECONDS of back-to-back launches,
-    # so that the clocks have ramped whatever --warmup says (a handful of 0.2 ms steps is over before
-    # the power management has reacted).
-    MIN_WARM_SECONDS = 0.25
-    done, t_w = 0, time.perf_counter()
-    while done < warmup or time.perf_counter() - t_w < MIN_WARM_SECONDS:
-        for _ in range(max(1, min(50, warmup - done))):
-            step(done)
-            done += 1
-        torch.cuda.synchronize()
-    warm_steps_run = done
-    # exactly `steps` timed steps; an event in front of every step (on the stream the kernels are
-    # launched on) gives the per-step times as well
-    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        evs[i].record()
-        step(i)
-    evs[steps].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    gpu_s = evs[0].elapsed_time(evs[steps]) * 1e-3
-    step_ms = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(steps))
+    wall, gpu_s, step_ms, warm_steps_run = timed_steps(step, steps, warmup)
     median_step_ms = step_ms[steps // 2]
 
     def abytes(K, N):
