@@ -129,8 +129,8 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   const __amdgpu_buffer_rsrc_t rcode = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<u4_t*>(P.codes + (size_t)slot_c * P.codes_slot_u4), 0, 0x7fffffff, 0x00020000);
   const int np_w = min(n0 / DZ_NPAIR + wave, P.NP - 1);
-  auto issue_delta = [&](int kb) {
-    unsigned char* dst = dstage + wave * DT;
+  auto issue_delta = [&](int kb, int stage = 0) {
+    unsigned char* dst = dstage + stage * (8 * DT) + wave * DT;
     const int tile = np_w * P.NKB + kb;
     const int lo = lane * 16;
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rmeta, (__attribute__((address_space(3))) void*)dst, 16, lo,
@@ -178,10 +178,87 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     issue_xd(1);
     issue_delta(0);
   };
-  if (nb > 0) issue(0, 0);
-  else if (nd > 0) delta_prologue();
-  // ---- base pass
-  for (int s = 0; s < nb; ++s) {
+  // ---- base weight and delta together: one walk over K.  Every slab is multiplied by the base
+  // weight (dense instruction) and by the delta's 64 columns (sparse instruction) from the same
+  // activation operands, read from LDS once; the delta's packed words are staged one k-block ahead
+  // as in the delta pass below.  A second walk would fetch every activation slab again and spend a
+  // barrier per slab on half as much matrix work.
+  constexpr bool FUSE = BITS == 2;   // (two staged k-blocks of 4-bit operands do not fit beside the slab buffers)
+  if (FUSE && nb > 0 && nd > 0) {
+    h2_t sc[4];
+    int scn[4];
+    issue(0, 0);
+    issue_delta(0, 0);
+    load_scales(scn, 0);
+    int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
+    for (int s = 0; s < nslab1; ++s) {
+      const int buf = s & 1, kb = s >> 2, j = s & 3;
+      __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): this wavefront's share of slab s (and of the staged k-block)
+      __syncthreads();
+      if (s + 1 < nslab1) issue(s + 1, buf ^ 1);
+      // the packed words of k-block kb sit in stage kb & 1 (each lane's words j of its four
+      // n-pairs are read from there slab by slab); the other stage, last read during k-block
+      // kb - 1, takes k-block kb + 1
+      if (j == 1 && kb + 1 < P.NKB) issue_delta(kb + 1, (kb + 1) & 1);
+      if (gleft == P.gslabs) spread_scales(sc, scn);
+      if (gleft == 1 && s + 1 < nslab1) load_scales(scn, gi + 1);
+      if (--gleft == 0) {
+        gleft = P.gslabs;
+        ++gi;
+      }
+      if (!has_rows) continue;
+      const unsigned char* wb = smem + buf * (2 * SLAB);
+      const unsigned char* xb = wb + SLAB;
+      // the activation operands of both halves stay in registers for the sparse product; the
+      // weight operands are taken four row tiles at a time (the accumulators leave little room)
+      h16_t B[4];
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const h8_t lo = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[0]);
+        const h8_t hi = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[1]);
+        B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+#pragma unroll
+        for (int ah = 0; ah < 2; ++ah) {
+          h8_t fw[4];
+#pragma unroll
+          for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + (4 * ah + a) * 16 * 128 + foff[h]);
+#pragma unroll
+          for (int b = 0; b < 4; ++b) {
+            const h8_t fxb = h == 0 ? __builtin_shufflevector(B[b], B[b], 0, 1, 2, 3, 4, 5, 6, 7)
+                                    : __builtin_shufflevector(B[b], B[b], 8, 9, 10, 11, 12, 13, 14, 15);
+#pragma unroll
+            for (int a = 0; a < 4; ++a)
+              acc[4 * ah + a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[a], fxb, acc[4 * ah + a][b], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);   // one group of weight operands at a time
+        }
+      const unsigned char* dsrc = dstage + (kb & 1) * (8 * DT) + (wn * 4) * DT + lane * 16 + j * 4;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const uint32_t mw = *(const uint32_t*)(dsrc + p * DT);
+        const uint32_t cw0 = *(const uint32_t*)(dsrc + p * DT + 1024);
+        h8_t A0, A1;
+        unpack2(cw0, MAGIC, A0, A1);
+        A0 *= sc[p][0];
+        A1 *= sc[p][1];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          acc[2 * p][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B[b], acc[2 * p][b], (int)mw, 0, 0);
+          acc[2 * p + 1][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B[b], acc[2 * p + 1][b], (int)mw, 0, 1);
+        }
+      }
+    }
+  }
+  const bool fused = FUSE && nb > 0 && nd > 0;
+  if (!fused) {
+    if (nb > 0) issue(0, 0);
+    else if (nd > 0) delta_prologue();
+  }
+  // ---- base pass (a block without a delta)
+  for (int s = 0; s < (fused ? 0 : nb); ++s) {
     const int buf = s & 1;
     // the slab of this turn was requested one turn ago: wait for this wavefront's share, then meet
     // the others (their shares are in, and nobody still reads the buffer filled next)
@@ -211,9 +288,9 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   Frag<BITS> cur[4];
   h2_t sc[4];
   int scn[4];
-  if (nd > 0) load_scales(scn, 0);
+  if (nd > 0 && !fused) load_scales(scn, 0);
   int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
-  for (int sd = 0; sd < nd; ++sd) {
+  for (int sd = 0; sd < (fused ? 0 : nd); ++sd) {
     const int kb = sd >> 2, j = sd & 3;
     // Slab sd was requested three turns ago (slabs 0 and 1: before the pass).  Loads complete in
     // order and at least the 8 requests of slabs sd + 1 and sd + 2 follow it, so "at most 8
@@ -375,7 +452,9 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
-  const size_t lds = 4 * SLAB + 8 * 3072;   // two base buffers = four ring stages, + staged k-block
+  // two slab buffers (= four ring stages of the delta pass) + the staged packed operands: one
+  // k-block of 8 n-pairs at 4 bits, two of them (the single walk over K alternates) at 2 bits
+  const size_t lds = 4 * SLAB + (bits == 2 ? 2 * 8 * 2048 : 8 * 3072);
   static std::atomic<unsigned long long> attr_done[2];
   auto go = [&](auto kern, int which) -> int {
     if (!dz_lds_limit_once(attr_done[which], (const void*)kern, (int)lds)) return DZ_ELAUNCH;
