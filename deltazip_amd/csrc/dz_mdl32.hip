@@ -223,7 +223,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
     // not order LDS reads after LDS-direct loads by itself.)
     {
-      constexpr int later = 2 * G * (BITS == 2 ? 2 : 3);
+      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + (PRE ? 2 : 0));   // both batches: words and, with PRE, scales
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
       // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
       // believes one outstanding, turns every later vmcnt wait into vmcnt(0)
