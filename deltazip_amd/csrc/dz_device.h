@@ -155,5 +155,5 @@ inline bool dz_lds_limit_once(std::atomic<unsigned long long>& done, const void*
 }
 
 // Launch of the T <= 32 kernel (dz_mdl32.hip).
-int dz_launch_mdl32(const MdlParams& P, int bits, bool pre, hipStream_t st, int ksplit_override);
-int dz_launch_mdl32_batch(const MdlParams* P, int nprob, int bits, bool pre, hipStream_t st, int ksplit_override);
+int dz_launch_mdl32(const MdlParams& P, int bits, int pre, hipStream_t st, int ksplit_override);
+int dz_launch_mdl32_batch(const MdlParams* P, int nprob, int bits, int pre, hipStream_t st, int ksplit_override);

@@ -691,7 +691,9 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     Q.tok0 = 0;
     Q.nchunk = 1;
   }
-  const bool pre = !(bits == 2 && gs == K);
+  // 0: 2-bit, one scale per row (applied to the sums); else scales applied to the operands, with
+  // one request (a k-block spans at most two groups) or two (groups of 64) per delta and k-block
+  const int pre = (bits == 2 && gs == K) ? 0 : (gs >= 128 ? 1 : 2);
   // 33..128 tokens: group the tokens by delta id on the device (no host round trip) and deal the
   // groups to the chunks of 32; one launch carries all chunks
   if (T > 32 && !order)

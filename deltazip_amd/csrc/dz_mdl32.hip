@@ -29,7 +29,7 @@ constexpr int WK32 = 4;
 constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is about a microsecond)
 
 // The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
-template <int BITS, int TT, bool PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, bool HAS_BASE>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
@@ -196,8 +196,9 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // (tokens) that belong to it.  The loader runs two batches ahead of the consumer.
     Frag<BITS> ring[2][G];
     // PRE: scales of the batch, one fp16 per lane and register: lane l holds row n0 + l%32 of the
-    // k-block's scale group l/32 (register 0) and l/32 + 2 (register 1); a step's scale reaches the
-    // lane that multiplies with it through a cross-lane move, not through memory
+    // k-block's scale group l/32 (register 0) and, when a k-block spans four groups (PRE == 2:
+    // groups of 64), l/32 + 2 (register 1); a step's scale reaches the lane that multiplies with it
+    // through a cross-lane move, not through memory
     unsigned rsc[2][G][2];
     unsigned long long ld_m = mdelta, use_m = mdelta;
     auto pop = [&](unsigned long long& m, int& kd, unsigned long long& cols) {
@@ -221,7 +222,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
           const int gb0 = (kb * DZ_KBLOCK) / P.gs + (ls >> 5);
           const _Float16* sb = P.scales + (size_t)(kd - 1) * P.scales_slot + n0 + (ls & 31);
           rs[g][0] = *(const unsigned short*)(sb + (size_t)min(gb0, P.G - 1) * P.N);
-          rs[g][1] = *(const unsigned short*)(sb + (size_t)min(gb0 + 2, P.G - 1) * P.N);
+          if (PRE == 2) rs[g][1] = *(const unsigned short*)(sb + (size_t)min(gb0 + 2, P.G - 1) * P.N);
         }
       }
     };
@@ -235,7 +236,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
     // not order LDS reads after LDS-direct loads by itself.)
     {
-      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + (PRE ? 2 : 0));   // both batches: words and, with PRE, scales
+      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + PRE);   // both batches: words and, with PRE, scales
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
       // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
       // believes one outstanding, turns every later vmcnt wait into vmcnt(0)
@@ -291,8 +292,11 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
               if (PRE) {
                 // the lane's operand rows are n0 + jj and n0 + 16 + jj; one scale per (row, K-group)
                 const int gk = (kb * DZ_KBLOCK + 64 * j) / P.gs - (kb * DZ_KBLOCK) / P.gs;   // 0..3
-                const unsigned pick = 0u - (unsigned)((gk >> 1) & 1);   // all ones: groups 2, 3
-                const int v = (int)((rs[g][1] & pick) | (rs[g][0] & ~pick));
+                int v = (int)rs[g][0];
+                if (PRE == 2) {
+                  const unsigned pick = 0u - (unsigned)((gk >> 1) & 1);   // all ones: groups 2, 3
+                  v = (int)((rs[g][1] & pick) | (rs[g][0] & ~pick));
+                }
                 const int src = (jj + ((gk & 1) << 5)) << 2;
                 const unsigned short s0 = (unsigned short)__builtin_amdgcn_ds_bpermute(src, v);
                 const unsigned short s1 = (unsigned short)__builtin_amdgcn_ds_bpermute(src + 64, v);
@@ -491,7 +495,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
 // that their partial sums can meet in that XCD's L2.  A launch may carry up to 4 chunks of 32 tokens
 // (33..128 tokens, grouped by delta id): the workgroups of the chunks of one (n-pair, k-chunk)
 // follow each other on the same XCD, so the base tile they all read comes from HBM once.
-template <int BITS, int TT, bool PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, bool HAS_BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
@@ -505,7 +509,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
 // would hold in one weight: q/k/v, gate/up) in one launch: the n-pairs of the calls are numbered
 // through, a workgroup picks its call by its n-pair.  One call's tail (reduction, stores) then
 // overlaps the next one's loads instead of leaving the memory system idle between launches.
-template <int BITS, int TT, bool PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, bool HAS_BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlBatch B) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
@@ -532,7 +536,7 @@ static int choose_split(const MdlParams& P, int np_total, int ksplit_override) {
 }
 
 template <int BITS, int TT>
-int launch32(MdlBatch B, int nprob, bool pre, hipStream_t st, int ksplit_override) {
+int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override) {
   // every call of a batch gets the split its n-pair count would get alone (the calls share K)
   int np_min = B.p[0].NP;
   for (int j = 1; j < nprob; ++j) np_min = B.p[j].NP < np_min ? B.p[j].NP : np_min;
@@ -553,20 +557,22 @@ int launch32(MdlBatch B, int nprob, bool pre, hipStream_t st, int ksplit_overrid
   }
   const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
-  static std::atomic<unsigned long long> attr_done[8];
+  static std::atomic<unsigned long long> attr_done[12];
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
-    const int which = slot + (nprob == 1 ? 0 : 4);
+    const int which = slot + (nprob == 1 ? 0 : 6);
     if (!dz_lds_limit_once(attr_done[which], f, (int)lds)) return DZ_ELAUNCH;
     if (nprob == 1) hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, B.p[0]);
     else hipLaunchKernelGGL(bkern, dim3(grid), dim3(64 * WK32), lds, st, B);
     return DZ_OK;
   };
   int rc;
-  if (pre) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, true, true>, dz_mdl32_batch_kernel<BITS, TT, true, true>, 0)
-                         : go(dz_mdl32_kernel<BITS, TT, true, false>, dz_mdl32_batch_kernel<BITS, TT, true, false>, 1);
-  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, false, true>, dz_mdl32_batch_kernel<BITS, TT, false, true>, 2)
-                     : go(dz_mdl32_kernel<BITS, TT, false, false>, dz_mdl32_batch_kernel<BITS, TT, false, false>, 3);
+  if (pre == 2) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 2, true>, dz_mdl32_batch_kernel<BITS, TT, 2, true>, 0)
+                              : go(dz_mdl32_kernel<BITS, TT, 2, false>, dz_mdl32_batch_kernel<BITS, TT, 2, false>, 1);
+  else if (pre == 1) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 1, true>, dz_mdl32_batch_kernel<BITS, TT, 1, true>, 2)
+                                   : go(dz_mdl32_kernel<BITS, TT, 1, false>, dz_mdl32_batch_kernel<BITS, TT, 1, false>, 3);
+  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 0, true>, dz_mdl32_batch_kernel<BITS, TT, 0, true>, 4)
+                     : go(dz_mdl32_kernel<BITS, TT, 0, false>, dz_mdl32_batch_kernel<BITS, TT, 0, false>, 5);
   if (rc) return rc;
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
@@ -575,7 +581,7 @@ int launch32(MdlBatch B, int nprob, bool pre, hipStream_t st, int ksplit_overrid
 
 // Launch of the fused kernel for one layer call or a batch of calls that share T, K, bits, the
 // scale grouping and the token order; called by dz_multi_delta_linear[_batch].
-int dz_launch_mdl32_batch(const MdlParams* P0, int nprob, int bits, bool pre, hipStream_t st, int ksplit_override) {
+int dz_launch_mdl32_batch(const MdlParams* P0, int nprob, int bits, int pre, hipStream_t st, int ksplit_override) {
   if (nprob < 1 || nprob > DZ_MAX_BATCH) return DZ_ESHAPE;
   MdlBatch B;
   for (int j = 0; j < DZ_MAX_BATCH; ++j) {
@@ -588,7 +594,7 @@ int dz_launch_mdl32_batch(const MdlParams* P0, int nprob, int bits, bool pre, hi
   return T <= 16 ? launch32<4, 1>(B, nprob, pre, st, ksplit_override) : launch32<4, 2>(B, nprob, pre, st, ksplit_override);
 }
 
-int dz_launch_mdl32(const MdlParams& P0, int bits, bool pre, hipStream_t st, int ksplit_override) {
+int dz_launch_mdl32(const MdlParams& P0, int bits, int pre, hipStream_t st, int ksplit_override) {
   return dz_launch_mdl32_batch(&P0, 1, bits, pre, st, ksplit_override);
 }
 
