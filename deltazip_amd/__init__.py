@@ -7,6 +7,7 @@ kernels for gfx950 behind the C ABI declared in include/dz_amd.h.  There is no C
 """
 from .checkpoint import (CompressionConfig, DeltaLayerWeights, DeltaModel, compress_model, convert_model,
                          save_compressed, save_converted)
+from .calibrate import lossy_compress
 from .config import DeltaConfig
 from .layers import (BaseLayerWithDelta, ColumnParallelLinearWithDelta, DeltaMapping, LogitsProcessorWithDelta,
                      MergedColumnParallelLinearWithDelta, MergedQKVParallelLinearWithDelta,
@@ -27,5 +28,5 @@ __all__ = [
     "DeltaLayerWeights", "DeltaModel", "convert_model", "compress_model", "save_compressed", "save_converted", "DeltaModelManager", "LRUCacheDeltaModelManager",
     "create_delta_manager", "LogitsProcessorWithDelta", "VocabParallelEmbeddingWithDelta",
     "from_layer_logits_processor", "apply_delta_embed", "apply_delta_uncompressed", "compress_delta", "apply_delta_batch", "token_order", "apply_delta_into", "apply_delta_packed_nslice",
-    "Quantizer", "SparseGPT",
+    "Quantizer", "SparseGPT", "lossy_compress",
 ]

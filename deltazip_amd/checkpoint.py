@@ -357,6 +357,14 @@ def compress_model(base_state_dict: Dict[str, torch.Tensor], target_state_dict: 
             native[key[: -len(".weight")]] = (q.cpu(), m.cpu(), s.cpu(), w.shape[1])
         elif key.endswith(".weight") and any(u in key for u in UNCOMPRESSED_MODULES):
             out[key if layout == "gptq" else key[: -len(".weight")] + ".0.weight"] = w.detach().cpu()
+    return _emit_state_dict(native, out, layout, pack_modules, bits, gs)
+
+
+def _emit_state_dict(native: Dict[str, Tuple[torch.Tensor, torch.Tensor, torch.Tensor, int]],
+                     out: Dict[str, torch.Tensor], layout: str, pack_modules: Dict[str, Tuple[str, int]],
+                     bits: int, gs: int) -> Dict[str, torch.Tensor]:
+    """Compressed modules {module: (qweight, meta, scales, K)} (native, unfused) + the uncompressed
+    entries already in `out` -> the state dict of the requested layout."""
     if layout == "gptq":
         for module, (q, m, s, K) in native.items():
             qw, qz, sc, gi = ops.unrepack_native_to_gptq(q, m, s, K, s.shape[-1], bits)
