@@ -154,6 +154,19 @@ inline bool dz_lds_limit_once(std::atomic<unsigned long long>& done, const void*
   return true;
 }
 
+// Compute units of the current device (looked up once per device).
+inline int dz_cu_count() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) return 256;
+  int v = cached[dev].load(std::memory_order_relaxed);
+  if (v == 0) {
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || v <= 0) v = 256;
+    cached[dev].store(v, std::memory_order_relaxed);
+  }
+  return v;
+}
+
 // Launch of the T <= 32 kernel (dz_mdl32.hip).
 int dz_launch_mdl32(const MdlParams& P, int bits, int pre, hipStream_t st, int ksplit_override);
 int dz_launch_mdl32_batch(const MdlParams* P, int nprob, int bits, int pre, hipStream_t st, int ksplit_override);

@@ -29,7 +29,7 @@ constexpr int WK32 = 4;
 constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is about a microsecond)
 
 // The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
-template <int BITS, int TT, int PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
@@ -105,7 +105,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // lane (ga, jj) fetches row 16*s + 8*half + jj % 8, 16-byte chunk 2*ga + jj / 8 of the step's 128
   // bytes.  The matrix instruction wants row jj in lane jj, so before use the upper eight lanes of
   // each group of 16 trade places between the two halves (`base_operands`).
-  auto issue_base = [&](int kb, int lane_r) {
+  auto issue_base = [&](int kb, int lane_r, const int s_lo, const int s_hi) {   // row fragments s_lo .. s_hi - 1
     const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
     const unsigned loff = (unsigned)(lane_r & 7) * Kb + (unsigned)(lane_r >> 4) * 32u + (unsigned)((lane_r >> 3) & 1) * 16u;
     // One chunk of tokens: the tile is read once in the whole launch and is requested as streaming
@@ -115,7 +115,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // when every chunk streams the tile for itself).
     if (P.nchunk > 1) {
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int s = s_lo; s < s_hi; ++s)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -123,7 +123,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
             a[s][j][h] = *(const u4_t*)(wbb + (size_t)(16 * s + 8 * h) * Kb + loff + 128 * j);
     } else {
 #pragma unroll
-      for (int s = 0; s < 2; ++s)
+      for (int s = s_lo; s < s_hi; ++s)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -166,7 +166,13 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     int lane_0 = lane;
     asm volatile("" : "+v"(lane_0));
     issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(id) : "n"(NX) : "memory");
+    // EARLY (launches of a single turn, where every workgroup starts on an idle memory system and
+    // would leave it idle until its ids are in): the first row fragment of the base tile, which
+    // does not depend on the ids, is requested right away.  In launches of several turns the later
+    // workgroups start while others stream, and the extra requests in front of the first batch of
+    // deltas cost as much as they gain there.
+    if (EARLY) issue_base(min(kb_lo + wave, P.NKB - 1), lane_0, 0, 1);
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(id) : "n"(NX + (EARLY ? 8 : 0)) : "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -179,7 +185,10 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     asm volatile("" : "+v"(lane_r));
 
     // the activations do not depend on the ids: they go first, the ids are awaited behind them
-    if (r > 0 && active) issue_x(kb, lane_r);
+    if (r > 0 && active) {
+      issue_x(kb, lane_r);
+      if (EARLY) issue_base(kb, lane_r, 0, 1);
+    }
     if (r == 0) {
       if (lane < Tc) {
         key = (id < 0 || id >= P.S) ? 0 : (int)id + 1;
@@ -236,7 +245,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
     // not order LDS reads after LDS-direct loads by itself.)
     {
-      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + PRE);   // both batches: words and, with PRE, scales
+      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + PRE) + (EARLY ? 8 : 0);   // both batches: words and, with PRE, scales; the early half of the base tile
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
       // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
       // believes one outstanding, turns every later vmcnt wait into vmcnt(0)
@@ -328,7 +337,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     consume(ring[0], rsc[0]);
     if (ld_m) load_batch(ring[0], rsc[0]);
     __builtin_amdgcn_sched_barrier(0);
-    if (HAS_BASE) issue_base(kb, lane_r);
+    if (HAS_BASE) issue_base(kb, lane_r, EARLY ? 1 : 0, 2);
     __builtin_amdgcn_sched_barrier(0);
     consume(ring[1], rsc[1]);
     if (ld_m) load_batch(ring[1], rsc[1]);
@@ -495,14 +504,14 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
 // that their partial sums can meet in that XCD's L2.  A launch may carry up to 4 chunks of 32 tokens
 // (33..128 tokens, grouped by delta id): the workgroups of the chunks of one (n-pair, k-chunk)
 // follow each other on the same XCD, so the base tile they all read comes from HBM once.
-template <int BITS, int TT, int PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
   const int per = P.nsplit * P.nchunk, rem = q % per;
   const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
   if (np >= P.NP) return;
-  mdl32_body<BITS, TT, PRE, HAS_BASE>(P, np, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, HAS_BASE, EARLY>(P, np, kc, ch, smem);
 }
 
 // Several layer calls that share tokens, K and the slot table (the projections a fused layer
@@ -519,7 +528,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlB
   // wavefront-uniform choice among the calls (np_end of unused entries repeats the total)
   const int j = (npg >= B.np_end[0]) + (npg >= B.np_end[1]) + (npg >= B.np_end[2]);
   const int first = j == 0 ? 0 : B.np_end[j - 1];
-  mdl32_body<BITS, TT, PRE, HAS_BASE>(B.p[j], npg - first, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, HAS_BASE, false>(B.p[j], npg - first, kc, ch, smem);
 }
 
 // K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
@@ -557,22 +566,28 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   }
   const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
-  static std::atomic<unsigned long long> attr_done[12];
+  // single launches of at most one turn (two workgroups per CU) take the variant that requests half
+  // the base tile before the ids are in
+  const bool early = nprob == 1 && has_base && grid <= 2 * dz_cu_count();
+  static std::atomic<unsigned long long> attr_done[15];
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
-    const int which = slot + (nprob == 1 ? 0 : 6);
-    if (!dz_lds_limit_once(attr_done[which], f, (int)lds)) return DZ_ELAUNCH;
+    if (!dz_lds_limit_once(attr_done[slot], f, (int)lds)) return DZ_ELAUNCH;
     if (nprob == 1) hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, B.p[0]);
     else hipLaunchKernelGGL(bkern, dim3(grid), dim3(64 * WK32), lds, st, B);
     return DZ_OK;
   };
-  int rc;
-  if (pre == 2) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 2, true>, dz_mdl32_batch_kernel<BITS, TT, 2, true>, 0)
-                              : go(dz_mdl32_kernel<BITS, TT, 2, false>, dz_mdl32_batch_kernel<BITS, TT, 2, false>, 1);
-  else if (pre == 1) rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 1, true>, dz_mdl32_batch_kernel<BITS, TT, 1, true>, 2)
-                                   : go(dz_mdl32_kernel<BITS, TT, 1, false>, dz_mdl32_batch_kernel<BITS, TT, 1, false>, 3);
-  else rc = has_base ? go(dz_mdl32_kernel<BITS, TT, 0, true>, dz_mdl32_batch_kernel<BITS, TT, 0, true>, 4)
-                     : go(dz_mdl32_kernel<BITS, TT, 0, false>, dz_mdl32_batch_kernel<BITS, TT, 0, false>, 5);
+  auto pick = [&](auto pre_c) -> int {
+    constexpr int PRE_ = decltype(pre_c)::value;
+    const int s0 = 5 * PRE_;
+    if (nprob > 1) return has_base ? go(dz_mdl32_kernel<BITS, TT, PRE_, true, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0)
+                                   : go(dz_mdl32_kernel<BITS, TT, PRE_, false, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, false>, s0 + 1);
+    if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, false, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, false>, s0 + 2);
+    return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, true, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0 + 3)
+                 : go(dz_mdl32_kernel<BITS, TT, PRE_, true, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0 + 4);
+  };
+  int rc = pre == 2 ? pick(std::integral_constant<int, 2>{}) : pre == 1 ? pick(std::integral_constant<int, 1>{})
+                                                                       : pick(std::integral_constant<int, 0>{});
   if (rc) return rc;
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
