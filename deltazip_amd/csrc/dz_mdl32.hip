@@ -546,10 +546,11 @@ static int choose_split(const MdlParams& P, int np_total, int ksplit_override) {
 
 template <int BITS, int TT>
 int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override) {
-  // every call of a batch gets the split its n-pair count would get alone (the calls share K)
-  int np_min = B.p[0].NP;
-  for (int j = 1; j < nprob; ++j) np_min = B.p[j].NP < np_min ? B.p[j].NP : np_min;
-  const int nsplit0 = choose_split(B.p[0], np_min, ksplit_override);
+  // K is split as far as the launch needs to fill the GPU: a batch counts the n-pairs of all its
+  // calls (gate + up together fill it without a split, and then exchange no partial sums at all)
+  int np_all = 0;
+  for (int j = 0; j < nprob; ++j) np_all += B.p[j].NP;
+  const int nsplit0 = choose_split(B.p[0], np_all, ksplit_override);
   int cb = (B.p[0].NKB + nsplit0 - 1) / nsplit0;
   cb = (cb + WK32 - 1) / WK32 * WK32;  // whole rounds
   const int nsplit = (B.p[0].NKB + cb - 1) / cb;

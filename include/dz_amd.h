@@ -217,8 +217,10 @@ int dz_multi_delta_linear_static(const uint16_t* x, const uint16_t* w_base,
  * MergedQKVParallelLinearWithDelta, gate/up: MergedColumnParallelLinearWithDelta,
  * serving/vllm/delta/layers_marlin.py:281-487) when their weights are separate tensors.  Call j
  * computes y[j][T, ldy[j]] (+)= x[j] @ w_base[j]^T + x[j] @ dequant(delta_j[indices])^T with
- * N[j] output features, exactly as dz_multi_delta_linear would; in one launch the reduction and
- * stores of one call overlap the loads of the next.  All calls have a base weight or none has.
+ * N[j] output features, as dz_multi_delta_linear would (the launch splits K by the output rows of
+ * all its calls together, so the fp32 partial sums over K may be added in another order than in a
+ * separate call: equal up to that rounding, and identical from run to run); in one launch the
+ * reduction and stores of one call overlap the loads of the next.  All calls have a base weight or none has.
  * order: NULL, or what dz_token_order wrote for these indices (then the grouping of the tokens is
  * not repeated: the reference, too, converts the mapping once per batch and every layer reuses
  * it, serving/vllm/delta/models.py:421-435).  workspace: dz_workspace_bytes(T, K, N[0] + ... +

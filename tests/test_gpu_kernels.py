@@ -453,12 +453,31 @@ def test_compressor_argument_checks(dev):
         ops.compress_delta(torch.zeros(32, 256), 4)
 
 
-@pytest.mark.parametrize("bits,gs,t,ns", [(2, -1, 32, (128, 128, 128)), (4, 128, 7, (64, 256)), (2, -1, 64, (96, 32, 32, 160)),
-                                          (4, -1, 128, (64, 64))])
-def test_batched_calls_equal_separate_calls(dev, bits, gs, t, ns):
+@pytest.mark.parametrize("bits,gs,t,ns,k", [(2, -1, 32, (128, 128, 128), 1024), (4, 128, 7, (64, 256), 1024),
+                                            (2, -1, 64, (96, 32, 32, 160), 1024), (4, -1, 128, (64, 64), 1024),
+                                            (2, -1, 32, (64, 96), 4096)])
+def test_batched_calls_equal_separate_calls(dev, bits, gs, t, ns, k):
     """Projections that share the tokens, in one launch: every output is bit for bit what the
-    separate call gives (same split of K, same order of additions), and matches the oracle."""
-    k, nd = 1024, 5
+    separate call gives when both split K the same way (1024 columns are never split; for 4096
+    the split is pinned, since a batch chooses it by the n-pairs of all its calls and the fp32
+    partial sums are then added in a different order), and matches the oracle."""
+    nd = 5
+    if k > 1024:
+        ops.set_ksplit(2)
+    try:
+        _batched_equal_separate(dev, bits, gs, t, ns, k, nd)
+    finally:
+        ops.set_ksplit(0)
+    if k > 1024:     # with the launch's own choice of split: equal within the parity bound
+        ps = [make_problem(n, k, bits, gs, nd, t, "uniform", 700 + 10 * j + n, dev) for j, n in enumerate(ns)]
+        ys = ops.apply_delta_batch(ps[0]["x"], [p["q"] for p in ps], [p["s"] for p in ps], [p["m"] for p in ps],
+                                   ps[0]["ids"], [p["wb"] for p in ps])
+        torch.cuda.synchronize()
+        for p, y in zip(ps, ys):
+            assert o.rel_err(y.cpu().numpy(), o.forward_ref(ps[0]["x_np"], p["wb_np"], p["dts"], ps[0]["ids_np"])) <= TOL
+
+
+def _batched_equal_separate(dev, bits, gs, t, ns, k, nd):
     ps = [make_problem(n, k, bits, gs, nd, t, "uniform", 700 + 10 * j + n, dev) for j, n in enumerate(ns)]
     ids = ps[0]["ids"]
     ids_np = ps[0]["ids_np"]
