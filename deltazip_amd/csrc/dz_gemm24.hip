@@ -5,18 +5,20 @@
 // One workgroup (8 wavefronts, two per SIMD) computes 256 output features x 256 tokens of one row
 // block; each wavefront owns 128 features x 64 tokens as 8 x 4 tiles of 16 x 16 (128 fp32
 // accumulators, in ordinary vector registers: the sparse instruction does not accumulate in the
-// accumulation registers).  K is walked
-// twice in slabs of 64 columns, into the same accumulators:
-//   base pass   weight slab and activation slab go from global memory straight into LDS (two
-//               buffers, the next slab is on its way while this one is multiplied);
-//               v_mfma_f32_16x16x32_f16.
-//   delta pass  the activation slab goes through LDS as before; the delta's packed codes and 2-bit
-//               positions (native layout: 16 bytes per lane per 32 x 256 tile, already in operand
-//               order) are staged one k-block ahead in the idle weight half of the LDS buffers,
-//               read back 16 bytes per lane, unpacked to fp16(scale * (q - zero)) -- the
-//               reference's rounding point, qlinear_cuda.py:306-308 -- and fed to the 2:4-sparse
-//               v_smfmac_f32_16x16x64_f16 together with their positions: half the matrix-core time
-//               of a dense product, and no dequantised copy of the delta ever exists in memory.
+// accumulation registers).  K is walked in slabs of 64 columns; weight slab and activation slab go
+// from global memory straight into LDS (two buffers, the next slab is on its way while this one is
+// multiplied).  The delta's packed codes and 2-bit positions (native layout: 16 bytes per lane per
+// 32 x 256 tile, already in operand order) are staged in LDS one k-block ahead, read back by the
+// lanes that use them, unpacked to fp16(scale * (q - zero)) -- the reference's rounding point,
+// qlinear_cuda.py:306-308 -- and fed to the 2:4-sparse v_smfmac_f32_16x16x64_f16 together with
+// their positions: half the matrix-core time of a dense product, and no dequantised copy of the
+// delta ever exists in memory.
+//   2-bit deltas  one walk: every slab is multiplied by the base weight (v_mfma_f32_16x16x32_f16)
+//                 and by the delta's 64 columns from the same activation operands; a block without
+//                 a delta, or a call without a base weight, skips the half it does not have.
+//   4-bit deltas  two walks into the same accumulators (two staged k-blocks of 4-bit words do not
+//                 fit beside the slab buffers): base pass, then a delta pass with the activations
+//                 in a ring of four stages.
 // Rows of x and y are addressed through an optional token order (the output of the segment sort),
 // so the batch is neither gathered nor scattered.
 #include <hip/hip_runtime.h>
@@ -95,13 +97,14 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   const __amdgpu_buffer_rsrc_t rx =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<_Float16*>(P.x), 0, 0x7fffffff, 0x00020000);
   // base pass: slab s -> buffer s & 1, [weight slab | activation slab]
-  auto issue = [&](int s, int buf) {
+  auto issue = [&](int s, int buf, bool with_w = true) {
     const int soff = s * (BK * 2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       unsigned char* dst = smem + buf * (2 * SLAB) + (wave * 4 + i) * 1024;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
-                                               (int)goff_w[i], soff, 0, 0);
+      if (with_w)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
+                                                 (int)goff_w[i], soff, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(dst + SLAB), 16,
                                                (int)goff_x[i], soff, 0, 0);
     }
@@ -178,33 +181,39 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     issue_xd(1);
     issue_delta(0);
   };
-  // ---- base weight and delta together: one walk over K.  Every slab is multiplied by the base
-  // weight (dense instruction) and by the delta's 64 columns (sparse instruction) from the same
-  // activation operands, read from LDS once; the delta's packed words are staged one k-block ahead
-  // as in the delta pass below.  A second walk would fetch every activation slab again and spend a
-  // barrier per slab on half as much matrix work.
+  // ---- 2-bit deltas: one walk over K for every kind of row block.  Every slab is multiplied by the
+  // base weight (dense instruction; skipped without a base weight) and by the delta's 64 columns
+  // (sparse instruction; skipped for a block without a delta) from the same activation operands,
+  // read from LDS once; the delta's packed words are staged one k-block ahead, alternating between
+  // two stages.  A second walk would fetch every activation slab again and spend a barrier per
+  // slab on half as much matrix work.
   constexpr bool FUSE = BITS == 2;   // (two staged k-blocks of 4-bit operands do not fit beside the slab buffers)
-  if (FUSE && nb > 0 && nd > 0) {
+  if constexpr (FUSE) {
+    const bool do_w = nb > 0, do_d = nd > 0;   // workgroup-uniform
     h2_t sc[4];
     int scn[4];
-    issue(0, 0);
-    issue_delta(0, 0);
-    load_scales(scn, 0);
+    if (total > 0) issue(0, 0, do_w);
+    if (do_d) {
+      issue_delta(0, 0);
+      load_scales(scn, 0);
+    }
     int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
-    for (int s = 0; s < nslab1; ++s) {
+    for (int s = 0; s < (total > 0 ? nslab1 : 0); ++s) {
       const int buf = s & 1, kb = s >> 2, j = s & 3;
       __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) lgkmcnt(0): this wavefront's share of slab s (and of the staged k-block)
       __syncthreads();
-      if (s + 1 < nslab1) issue(s + 1, buf ^ 1);
-      // the packed words of k-block kb sit in stage kb & 1 (each lane's words j of its four
-      // n-pairs are read from there slab by slab); the other stage, last read during k-block
-      // kb - 1, takes k-block kb + 1
-      if (j == 1 && kb + 1 < P.NKB) issue_delta(kb + 1, (kb + 1) & 1);
-      if (gleft == P.gslabs) spread_scales(sc, scn);
-      if (gleft == 1 && s + 1 < nslab1) load_scales(scn, gi + 1);
-      if (--gleft == 0) {
-        gleft = P.gslabs;
-        ++gi;
+      if (s + 1 < nslab1) issue(s + 1, buf ^ 1, do_w);
+      if (do_d) {
+        // the packed words of k-block kb sit in stage kb & 1 (each lane's words j of its four
+        // n-pairs are read from there slab by slab); the other stage, last read during k-block
+        // kb - 1, takes k-block kb + 1
+        if (j == 1 && kb + 1 < P.NKB) issue_delta(kb + 1, (kb + 1) & 1);
+        if (gleft == P.gslabs) spread_scales(sc, scn);
+        if (gleft == 1 && s + 1 < nslab1) load_scales(scn, gi + 1);
+        if (--gleft == 0) {
+          gleft = P.gslabs;
+          ++gi;
+        }
       }
       if (!has_rows) continue;
       const unsigned char* wb = smem + buf * (2 * SLAB);
@@ -222,6 +231,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       for (int h = 0; h < 2; ++h)
 #pragma unroll
         for (int ah = 0; ah < 2; ++ah) {
+          if (!do_w) break;
           h8_t fw[4];
 #pragma unroll
           for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + (4 * ah + a) * 16 * 128 + foff[h]);
@@ -238,6 +248,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       const unsigned char* dsrc = dstage + (kb & 1) * (8 * DT) + (wn * 4) * DT + lane * 16 + j * 4;
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
+        if (!do_d) break;
         const uint32_t mw = *(const uint32_t*)(dsrc + p * DT);
         const uint32_t cw0 = *(const uint32_t*)(dsrc + p * DT + 1024);
         h8_t A0, A1;
@@ -252,13 +263,11 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       }
     }
   }
-  const bool fused = FUSE && nb > 0 && nd > 0;
-  if (!fused) {
-    if (nb > 0) issue(0, 0);
-    else if (nd > 0) delta_prologue();
-  }
-  // ---- base pass (a block without a delta)
-  for (int s = 0; s < (fused ? 0 : nb); ++s) {
+  if constexpr (!FUSE) {
+  // ---- 4-bit deltas: base pass, then delta pass
+  if (nb > 0) issue(0, 0);
+  else if (nd > 0) delta_prologue();
+  for (int s = 0; s < nb; ++s) {
     const int buf = s & 1;
     // the slab of this turn was requested one turn ago: wait for this wavefront's share, then meet
     // the others (their shares are in, and nobody still reads the buffer filled next)
@@ -288,9 +297,9 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   Frag<BITS> cur[4];
   h2_t sc[4];
   int scn[4];
-  if (nd > 0 && !fused) load_scales(scn, 0);
+  if (nd > 0) load_scales(scn, 0);
   int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
-  for (int sd = 0; sd < (fused ? 0 : nd); ++sd) {
+  for (int sd = 0; sd < nd; ++sd) {
     const int kb = sd >> 2, j = sd & 3;
     // Slab sd was requested three turns ago (slabs 0 and 1: before the pass).  Loads complete in
     // order and at least the 8 requests of slabs sd + 1 and sd + 2 follow it, so "at most 8
@@ -368,6 +377,8 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       }
     }
   }
+
+  }   // 4-bit passes
 
   // ---- store: lane (i, g) holds features 4*g .. 4*g + 3 of tile a for token i of tile b
 #pragma unroll
