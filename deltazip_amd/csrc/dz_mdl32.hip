@@ -552,7 +552,8 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   for (int j = 0; j < nprob; ++j) np_all += B.p[j].NP;
   const int nsplit0 = choose_split(B.p[0], np_all, ksplit_override);
   int cb = (B.p[0].NKB + nsplit0 - 1) / nsplit0;
-  cb = (cb + WK32 - 1) / WK32 * WK32;  // whole rounds
+  // (K-slices need not be whole rounds of WK32 k-blocks: a wavefront without a k-block in a
+  // slice's last round idles; rounding the slice length up leaves the last slice short instead)
   const int nsplit = (B.p[0].NKB + cb - 1) / cb;
   int np_total = 0;
   bool has_base = B.p[0].wb != nullptr;
