@@ -150,29 +150,71 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // of the loop over k-blocks.
   int key = 0x7fffffff;
   unsigned long long mdelta = 0;
-  // The ids are requested before anything else and nothing more is requested until they are in:
-  // a request queued behind this kernel's own flood of weight loads takes several microseconds.
+  // Nothing from HBM can be requested before the token ids are in (which deltas to fetch depends
+  // on them), and a request queued behind this kernel's own flood of weight loads takes several
+  // microseconds: the ids go out with the round's activations (L2 hits) and are awaited with them.
+  // They are requested outside the compiler's bookkeeping -- it would wait for every LDS-direct
+  // load in flight, being unable to tell them apart -- which needs care: the compiler takes the
+  // destination register of an asm statement for valid the moment the statement ends and is free
+  // to spill or copy it while the load is still in flight.  So either the load and its wait sit in
+  // one statement, or the ids go to LDS and no register is involved until they are read back.
   long long id = -1;
-  if (lane < Tc) {
-    prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
-    const long long* ip = P.idx + prow;
-    // requested outside the compiler's bookkeeping: it would wait for the LDS-direct loads that
-    // follow as well (it cannot tell them apart); the wait below counts them instead
-    asm volatile("global_load_dwordx2 %0, %1, off" : "+v"(id) : "v"(ip) : "memory");
-  }
-  __builtin_amdgcn_sched_barrier(0);
-  {
-    // round 0's activations (a wavefront without a k-block fetches a slice it will not use)
-    int lane_0 = lane;
-    asm volatile("" : "+v"(lane_0));
-    issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
-    // EARLY (launches of a single turn, where every workgroup starts on an idle memory system and
-    // would leave it idle until its ids are in): the first row fragment of the base tile, which
-    // does not depend on the ids, is requested right away.  In launches of several turns the later
-    // workgroups start while others stream, and the extra requests in front of the first batch of
-    // deltas cost as much as they gain there.
-    if (EARLY) issue_base(min(kb_lo + wave, P.NKB - 1), lane_0, 0, 1);
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(id) : "n"(NX + (EARLY ? 8 : 0)) : "memory");
+  if constexpr (EARLY) {
+    // Launches of a single turn: every workgroup starts on an idle memory system and would leave
+    // it idle until its ids are in, so the first row fragment of the base tile, which does not
+    // depend on the ids, is requested right away.  (In launches of several turns the later
+    // workgroups start while others stream, and extra requests in front of the first batch of
+    // deltas cost as much as they gain there.)  Order: ids -> LDS, activations, half the base tile;
+    // then "at most NX + 8 requests outstanding" means the ids have arrived.  LDS layout of the ids:
+    // 64 low words, 64 high words, behind the activation slices.
+    const unsigned id_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem +
+                            (unsigned)(WK32 * TP * DZ_KBLOCK * 2 + wave * 512);
+    if (lane < Tc) {
+      prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
+      const char* ip = (const char*)(P.idx + prow);
+      asm volatile(
+          "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %2, off\n\t"
+          "s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %3, off"
+          :
+          : "s"(id_lds), "s"(id_lds + 256u), "v"(ip), "v"(ip + 4)
+          : "memory", "m0");
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      // round 0's activations (a wavefront without a k-block fetches a slice it will not use)
+      int lane_0 = lane;
+      asm volatile("" : "+v"(lane_0));
+      issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
+      issue_base(min(kb_lo + wave, P.NKB - 1), lane_0, 0, 1);
+      // nothing of the compiler's between the two waits: a scalar load scheduled in there would
+      // be waited for by the lgkmcnt(0) below instead of behind the ids' latency
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NX + 8) : "memory");
+    }
+    {
+      unsigned lo, hi;   // read and wait in one statement
+      asm volatile("ds_read_b32 %0, %2\n\tds_read_b32 %1, %2 offset:256\n\ts_waitcnt lgkmcnt(0)"
+                   : "=&v"(lo), "=&v"(hi)
+                   : "v"(id_lds + 4u * (unsigned)lane)
+                   : "memory");
+      if (lane < Tc) id = (long long)(((unsigned long long)hi << 32) | lo);
+    }
+  } else {
+    // Activations first, then the ids and the wait for everything so far in one statement: the
+    // ids return behind the activations, which are L2 hits and long in by then.
+    const char* ip = nullptr;
+    if (lane < Tc) {
+      prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
+      ip = (const char*)(P.idx + prow);
+    }
+    {
+      int lane_0 = lane;
+      asm volatile("" : "+v"(lane_0));
+      issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (lane < Tc)
+      asm volatile("global_load_dwordx2 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "+v"(id) : "v"(ip) : "memory");
   }
   __builtin_amdgcn_sched_barrier(0);
 
@@ -567,7 +609,7 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
     B.np_end[j] = np_total;
   }
   const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
-  const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2;
+  const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2 + WK32 * 512;   // activation slices + the token ids
   // single launches of at most one turn (two workgroups per CU) take the variant that requests half
   // the base tile before the ids are in
   const bool early = nprob == 1 && has_base && grid <= 2 * dz_cu_count();

@@ -455,7 +455,12 @@ def test_compressor_argument_checks(dev):
 
 @pytest.mark.parametrize("bits,gs,t,ns,k", [(2, -1, 32, (128, 128, 128), 1024), (4, 128, 7, (64, 256), 1024),
                                             (2, -1, 64, (96, 32, 32, 160), 1024), (4, -1, 128, (64, 64), 1024),
-                                            (2, -1, 32, (64, 96), 4096)])
+                                            (2, -1, 32, (64, 96), 4096),
+                                            # 2-bit deltas with scale groups of 64: the kernel variant under the
+                                            # highest register pressure (it once spilled a register that an
+                                            # in-flight load was still to fill)
+                                            (2, 64, 32, (160, 160), 1024), (2, 64, 102, (96, 96), 768),
+                                            (2, 64, 65, (32, 32), 4096), (2, 64, 7, (64, 32), 512)])
 def test_batched_calls_equal_separate_calls(dev, bits, gs, t, ns, k):
     """Projections that share the tokens, in one launch: every output is bit for bit what the
     separate call gives when both split K the same way (1024 columns are never split; for 4096
