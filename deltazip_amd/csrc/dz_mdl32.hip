@@ -33,7 +33,7 @@ template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
-  constexpr int G = (BITS == 2) ? 4 : (TT == 2 ? 2 : 3);   // deltas per batch; two batches are in flight
+  constexpr int G = (BITS == 2) ? (PRE == 2 ? 3 : 4) : (TT == 2 ? 2 : 3);   // deltas per batch (two batches are in flight); 3 where 4 would not fit the registers
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform, in a scalar register
