@@ -40,13 +40,24 @@ def build_library(verbose: bool = False, extra_flags=()) -> str:
         err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
         if res.returncode != 0:
             raise RuntimeError("hipcc failed:\n" + err)
-        if verbose and err.strip():
-            print(err, file=sys.stderr)
+        return err
 
     def compile_one(src):
         obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
-        run([hipcc, *[f for f in HIPCC_FLAGS if f != "-shared"], *extra_flags, "-x", "hip", "-c",
-             os.path.join(CSRC, src), "-o", obj])
+        err = run([hipcc, *[f for f in HIPCC_FLAGS if f != "-shared"], *extra_flags,
+                   "-Rpass-analysis=kernel-resource-usage", "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj])
+        # The kernels are written to fit the register file: a variant that starts to use scratch
+        # memory (register spills) has lost the performance it was tuned for.  Say so at build time.
+        name, rest = None, []
+        for line in err.splitlines():
+            if "remark:" not in line:
+                rest.append(line)
+            elif "Function Name:" in line:
+                name = line.split("Function Name:")[1].split("[")[0].strip()
+            elif "ScratchSize [bytes/lane]:" in line and int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0]) > 0:
+                print(f"warning: {src}: kernel {name} uses scratch memory", file=sys.stderr)
+        if verbose and "\n".join(rest).strip():
+            print("\n".join(rest), file=sys.stderr)
         return obj
 
     with ThreadPoolExecutor(max_workers=min(len(srcs), os.cpu_count() or 4)) as pool:
