@@ -421,6 +421,17 @@ def _infer(qweight_stacked, scales_stacked, N: int):
     return S, words, G
 
 
+def takes_fused_chunks(T: int, S: int) -> bool:
+    """Whether a batch above the fused kernel's 128 tokens goes through it in chunks of 128 rather than
+    through the matrix-core kernel.  That kernel works on row blocks of up to 256 tokens of one delta
+    and needs some 256 x (N / 256) of them to fill the GPU: a few hundred tokens, the more so when
+    they are spread over many deltas, leave most of it idle (5120 x 5120, 2-bit, 256 tokens: 0.13 to
+    0.19 ms in two chunks against 0.18 ms with one delta and 0.57 ms with 64; at 1024 tokens the
+    matrix cores win unless every 16 tokens belong to another delta).  The number of distinct deltas
+    is known on the device only, so the number of slots stands in for it."""
+    return T <= 2 * MAX_TOKENS_FUSED or (T <= 4 * MAX_TOKENS_FUSED and S >= 32)
+
+
 def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qweight_stacked,
                        scales_stacked, meta_stacked, indices: torch.Tensor, *, bits: int,
                        out: Optional[torch.Tensor] = None, accumulate: bool = False,
@@ -465,6 +476,12 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
             raise ValueError("out must be float16 [T, N] with unit column stride")
     ldy = out.stride(0)
     if T > MAX_TOKENS_FUSED:
+        if takes_fused_chunks(T, S):
+            for r in range(0, T, MAX_TOKENS_FUSED):
+                multi_delta_linear(x2[r:r + MAX_TOKENS_FUSED], base_weight, qweight_stacked, scales_stacked,
+                                   meta_stacked, indices[r:r + MAX_TOKENS_FUSED], bits=bits,
+                                   out=out[r:r + MAX_TOKENS_FUSED], accumulate=accumulate)
+            return out
         from .prefill import multi_delta_linear_prefill
         return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
                                           indices, bits=bits, out=out, accumulate=accumulate)

@@ -274,6 +274,29 @@ def test_prefill_sized_call(dev, kind):
     assert o.rel_err(y, ref) <= TOL
 
 
+@pytest.mark.parametrize("t,nd", [(129, 3), (256, 40), (300, 40), (512, 33)])
+def test_mid_size_batches_go_through_the_fused_kernel_in_chunks(dev, t, nd):
+    """Between 129 tokens and a few hundred the matrix-core kernel would leave most of the GPU idle:
+    the call is made of chunks of 128 tokens through the fused kernel.  Both routes match the oracle."""
+    from deltazip_amd.prefill import multi_delta_linear_prefill
+    assert ops.takes_fused_chunks(t, nd) and not ops.takes_fused_chunks(513, 64) and not ops.takes_fused_chunks(300, 4)
+    p = make_problem(96, 512, 2, -1, nd, t, "uniform", 77 + t, dev)
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    y = run_layer(p)
+    assert o.rel_err(y.cpu().numpy(), ref) <= TOL
+    y2 = torch.empty_like(y)
+    multi_delta_linear_prefill(p["x"], p["wb"], p["q"], p["s"], p["m"], p["ids"], bits=2, out=y2, accumulate=False)
+    torch.cuda.synchronize()
+    assert o.rel_err(y2.cpu().numpy(), ref) <= TOL
+    # in place, delta only, into a column slice: the chunks write their rows of the slice
+    wide = torch.zeros(t, 96 + 64, device=dev, dtype=torch.float16)
+    ops.add_delta_slice(wide, p["x"], p["q"], None, p["s"], None, p["ids"], 1.0, 32, 96, meta=p["m"])
+    torch.cuda.synchronize()
+    dref = ref - p["x_np"].astype(np.float32) @ p["wb_np"].astype(np.float32).T
+    assert float(wide[:, :32].abs().max()) == 0 and float(wide[:, 128:].abs().max()) == 0
+    assert np.abs(wide[:, 32:128].float().cpu().numpy() - dref).max() <= 2e-2 * np.abs(dref).max()
+
+
 def test_gemm_grouped(dev):
     """Grouped GEMM through the C ABI: ragged row blocks, a block without second weight, rows that no
     block covers (left untouched), an N that is not a multiple of the 256-wide tile, and the
