@@ -29,7 +29,7 @@ constexpr int WK32 = 4;
 constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is about a microsecond)
 
 // The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
-template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY>
+template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY, bool IDL>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
@@ -156,17 +156,18 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // They are requested outside the compiler's bookkeeping -- it would wait for every LDS-direct
   // load in flight, being unable to tell them apart -- which needs care: the compiler takes the
   // destination register of an asm statement for valid the moment the statement ends and is free
-  // to spill or copy it while the load is still in flight.  So either the load and its wait sit in
-  // one statement, or the ids go to LDS and no register is involved until they are read back.
+  // to spill or copy it while the load is still in flight.  So either the ids go to LDS and no
+  // register is involved until they are read back (IDL: launches of one call), or the load and its
+  // wait sit in one statement (the batched launches, where the first way measured 1 % slower).
   long long id = -1;
-  if constexpr (EARLY) {
-    // Launches of a single turn: every workgroup starts on an idle memory system and would leave
-    // it idle until its ids are in, so the first row fragment of the base tile, which does not
-    // depend on the ids, is requested right away.  (In launches of several turns the later
-    // workgroups start while others stream, and extra requests in front of the first batch of
-    // deltas cost as much as they gain there.)  Order: ids -> LDS, activations, half the base tile;
-    // then "at most NX + 8 requests outstanding" means the ids have arrived.  LDS layout of the ids:
-    // 64 low words, 64 high words, behind the activation slices.
+  if constexpr (IDL) {
+    // Order: ids -> LDS, activations, then (EARLY) half the base tile; "at most NX (+ 8) requests
+    // outstanding" then means the ids have arrived.  EARLY, launches of a single turn: every
+    // workgroup starts on an idle memory system and would leave it idle until its ids are in, so
+    // the first row fragment of the base tile, which does not depend on the ids, is requested right
+    // away.  (In launches of several turns the later workgroups start while others stream, and
+    // extra requests in front of the first batch of deltas cost as much as they gain there.)
+    // LDS layout of the ids: 64 low words, 64 high words, behind the activation slices.
     const unsigned id_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem +
                             (unsigned)(WK32 * TP * DZ_KBLOCK * 2 + wave * 512);
     if (lane < Tc) {
@@ -185,11 +186,11 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
       int lane_0 = lane;
       asm volatile("" : "+v"(lane_0));
       issue_x(min(kb_lo + wave, P.NKB - 1), lane_0);
-      issue_base(min(kb_lo + wave, P.NKB - 1), lane_0, 0, 1);
+      if (EARLY) issue_base(min(kb_lo + wave, P.NKB - 1), lane_0, 0, 1);
       // nothing of the compiler's between the two waits: a scalar load scheduled in there would
       // be waited for by the lgkmcnt(0) below instead of behind the ids' latency
       __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NX + 8) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NX + (EARLY ? 8 : 0)) : "memory");
     }
     {
       unsigned lo, hi;   // read and wait in one statement
@@ -553,7 +554,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams 
   const int per = P.nsplit * P.nchunk, rem = q % per;
   const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
   if (np >= P.NP) return;
-  mdl32_body<BITS, TT, PRE, HAS_BASE, EARLY>(P, np, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, HAS_BASE, EARLY, true>(P, np, kc, ch, smem);
 }
 
 // Several layer calls that share tokens, K and the slot table (the projections a fused layer
@@ -570,7 +571,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlB
   // wavefront-uniform choice among the calls (np_end of unused entries repeats the total)
   const int j = (npg >= B.np_end[0]) + (npg >= B.np_end[1]) + (npg >= B.np_end[2]);
   const int first = j == 0 ? 0 : B.np_end[j - 1];
-  mdl32_body<BITS, TT, PRE, HAS_BASE, false>(B.p[j], npg - first, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, HAS_BASE, false, false>(B.p[j], npg - first, kc, ch, smem);
 }
 
 // K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
