@@ -39,9 +39,9 @@ T, NUM_DELTAS, BITS, GROUP = 32, 8, 2, -1    # the default workload (configurati
 # measured on: it is reported only while their fingerprint (kernel_fingerprint) still equals the
 # one recorded here with the profile, and withheld (null) once the kernel has changed.
 MEASURED_TRAFFIC = {
-    "bytes_per_launch": 213080817,
+    "bytes_per_launch": 212929225,
     "profile": "profiles/dz_mdl32_kernel__llama7b_decode_t32_d8_2bit__hbm_traffic.txt",
-    "kernel_sha256": "108b843a0ecf96d6a22993ff60b6372cb8d4669ba6877897b6c5592fd5b089ba",
+    "kernel_sha256": "a54c0f3a70e9ab1da8a7ad318108d8bfb89e8f1f1a8f9156d92f9f00e2fd5a82",
 }
 KERNEL_SOURCES = ("deltazip_amd/csrc/dz_mdl32.hip", "deltazip_amd/csrc/dz_device.h", "deltazip_amd/csrc/dz_layout.h")
 
@@ -78,10 +78,14 @@ def parity_check(dev):
                                np.ascontiguousarray(dts[d].T).view(np.uint16)) for d in range(nd))
     wb, x = o.make_base(n, k, 2000), o.make_x(T, k, 2500)
     ids = np.sort(o.make_ids("uniform", T, nd, 2900))
-    y = ops.apply_delta(torch.from_numpy(x).to(dev), q, s, m, torch.from_numpy(ids).to(dev), torch.from_numpy(wb).to(dev))
-    err = o.rel_err(y.cpu().numpy(), o.forward_ref(x, wb, dts, ids))
+    xd, idd, wbd = torch.from_numpy(x).to(dev), torch.from_numpy(ids).to(dev), torch.from_numpy(wb).to(dev)
+    ref = o.forward_ref(x, wb, dts, ids)
+    y = ops.apply_delta(xd, q, s, m, idd, wbd)
+    yt = ops.apply_delta(xd, q, s, m, idd, wbd, base_tiled=ops.tile_base(wbd))   # the form the timed loop reads
+    err = max(o.rel_err(y.cpu().numpy(), ref), o.rel_err(yt.cpu().numpy(), ref))
+    same = bool(torch.equal(y, yt))
     return {"dequant_bit_exact": bool(exact), "max_rel_err": float(err), "tolerance": 1e-2,
-            "ok": bool(exact and err <= 1e-2)}
+            "tiled_base_equals_row_major": same, "ok": bool(exact and same and err <= 1e-2)}
 
 
 def _cpu_model():
@@ -233,7 +237,8 @@ def run_full_step(args, parity):
     mcfg = LlamaStepConfig(num_hidden_layers=args.layers or 32)
     model = LlamaForDecodeStep(mcfg, device=dev, generator=gen)
     mgr = create_delta_manager(model, max_num_seqs=T, max_num_batched_tokens=T, vocab_size=mcfg.vocab_size,
-                               delta_config=DeltaConfig(max_deltas=S, max_bitwidth=bits, group_size=gs))
+                               delta_config=DeltaConfig(max_deltas=S, max_bitwidth=bits, group_size=gs,
+                                                        tile_base_weights=not args.row_major_base))
     # synthetic deltas written straight into the layers' slot stacks (compressing 64 x 32 real deltas
     # would take hours); the manager is told that delta d + 1 lives in slot d
     for name, layer in mgr.modules.items():
@@ -271,7 +276,9 @@ def run_full_step(args, parity):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": cfg["name"] + ", batch sorted by delta id", "baseline_config": 5, "tokens": T,
                    "deltas": S, "deltas_present": d_present, "bits": bits, "group_size": gs, "kv_context": ctx,
-                   "layers": mcfg.num_hidden_layers, "launches_per_step": len(projs)},
+                   "layers": mcfg.num_hidden_layers, "launches_per_step": len(projs),
+                   "base_weight_layout": "row-major [N, K]" if args.row_major_base
+                                         else "tiles (dz_tile_base, converted once when the layer is created)"},
         "linear_layers": {"ms_per_step": round(lin_ms, 4), "share_of_step": round(lin_ms / (gpu_s / steps * 1e3), 4),
                           "calls": len(projs), "us_per_call": round(lin_ms * 1e3 / len(projs), 2)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -293,6 +300,9 @@ def main():
     ap.add_argument("--layers", type=int, default=0, help="distinct decoder layers kept in HBM and visited in turn "
                                                        "(--config 5: decoder layers of the model, default 32)")
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
+    ap.add_argument("--row-major-base", action="store_true",
+                    help="up to 128 tokens: read the base weight as the plain [N, K] tensor instead of the tiled copy "
+                         "a layer makes of it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--ksplit", type=int, default=0)
     ap.add_argument("--separate-launches", action="store_true",
@@ -325,6 +335,9 @@ def main():
         return run_full_step(args, parity)
 
     # ---- resident inputs
+    # up to 128 tokens the layer reads its base weight from the tiled copy it makes at creation
+    # (dz_tile_base); --row-major-base measures the fused kernel on the plain [N, K] weight instead
+    tiled_base = T <= 128 and not args.row_major_base
     ids = make_ids(cfg["ids"], T, S, dev, gen, not args.unsorted)
     d_present = int(torch.unique(ids).numel())
     layers = []
@@ -333,6 +346,8 @@ def main():
         for name, K, N in shapes:
             q, m, s = random_native_stack(K, N, bits, gs, S, dev, gen)
             wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
+            if tiled_base:
+                wb = ops.tile_base(wb)      # as a layer does once when it is created; only this form is read
             x = torch.randn((T, K), device=dev, generator=gen).half()
             y = torch.empty((T, N), dtype=torch.float16, device=dev)
             calls.append((name, K, N, x, wb, q, m, s, y))
@@ -352,7 +367,8 @@ def main():
         # pre-marshalled C-ABI calls (device pointers and sizes only)
         ws_bytes = max(lib.dz_workspace_bytes(T, shapes[g[0]][1], sum(shapes[j][2] for j in g)) for g in groups)
         ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-        f, fb = lib.dz_multi_delta_linear, lib.dz_multi_delta_linear_batch
+        f = lib.dz_multi_delta_linear
+        fb = lib.dz_multi_delta_linear_batch_tiled if tiled_base else lib.dz_multi_delta_linear_batch
         vp = C.c_void_p
         # 33..128 tokens: the order in which the kernel takes the tokens depends on the ids only; it is
         # computed once per step (inside the timed region) and every launch of the step reuses it, as the
@@ -364,7 +380,7 @@ def main():
         for calls in layers:
             pc = []
             for g in groups:
-                if len(g) == 1 and order is None:
+                if len(g) == 1 and order is None and not tiled_base:
                     name, K, N, x, wb, q, m, s, y = calls[g[0]]
                     pc.append((f, (vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()),
                                    vp(s.data_ptr()), vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
@@ -379,10 +395,20 @@ def main():
                                     gs, 0, vp(order.data_ptr()) if order is not None else None,
                                     vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))))
             prepared.append(pc)
-            single.append([(vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
-                            vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
-                            vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))
-                           for name, K, N, x, wb, q, m, s, y in calls])
+            if tiled_base:
+                one = []
+                for name, K, N, x, wb, q, m, s, y in calls:
+                    a1 = [(vp * 1)(t.data_ptr()) for t in (x, wb, q, m, s, y)]
+                    an = (C.c_int * 1)(N)
+                    keep.append((a1, an))
+                    one.append((1, a1[0], a1[1], a1[2], a1[3], a1[4], vp(ids.data_ptr()), a1[5], an, an, T, K, S, bits, gs, 0,
+                                None, vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream)))
+                single.append(one)
+            else:
+                single.append([(vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
+                                vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
+                                vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))
+                               for name, K, N, x, wb, q, m, s, y in calls])
 
         def launch(i, gi):
             fn, a = prepared[i % len(prepared)][gi]
@@ -391,7 +417,7 @@ def main():
                 raise RuntimeError(f"multi-delta linear launch failed: {lib.dz_strerror(rc).decode()}")
 
         def call(i, idx):
-            rc = f(*single[i % len(single)][idx])
+            rc = (fb if tiled_base else f)(*single[i % len(single)][idx])
             if rc:
                 raise RuntimeError(f"dz_multi_delta_linear failed: {lib.dz_strerror(rc).decode()}")
     else:
@@ -424,7 +450,8 @@ def main():
 
     def abytes(K, N):
         return algorithmic_bytes(K, N, T, bits, d_present, 1 if gs == -1 else K // gs)
-    default_workload = args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
+    default_workload = (args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
+                        and not args.row_major_base)
     launches = steps * len(groups)
     step_bytes = sum(abytes(K, N) for _, K, N in shapes)
     step_flops = sum(2.0 * T * K * N for _, K, N in shapes)
@@ -481,7 +508,9 @@ def main():
                                               else ", batch sorted by delta id"),
                    "baseline_config": args.config, "tokens": T, "deltas": S, "deltas_present": d_present,
                    "bits": bits, "group_size": gs, "layers_resident": nlayers, "launches_per_step": len(groups),
-                   "launches": ["+".join(names[j] for j in g) for g in groups]},
+                   "launches": ["+".join(names[j] for j in g) for g in groups],
+                   "base_weight_layout": "tiles (dz_tile_base, converted once like the deltas)" if tiled_base
+                                         else "row-major [N, K]"},
         "us_per_layer_call": round(gpu_s / (steps * len(shapes)) * 1e6, 2),
         "per_shape": per_call_us,
         "roofline": roofline,

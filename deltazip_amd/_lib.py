@@ -33,6 +33,9 @@ SIGNATURES = {
     "dz_obs_sweep": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "dz_multi_delta_linear_batch": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp,
                                          _vp, C.c_size_t, _vp]),
+    "dz_multi_delta_linear_batch_tiled": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i,
+                                               _vp, _vp, C.c_size_t, _vp]),
+    "dz_tile_base": (_i, [_vp, _i, _i, _vp, _vp]),
     "dz_token_order": (_i, [_vp, _i, _i, _vp, _vp]),
     "dz_map_ids": (_i, [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "dz_workspace_bytes": (_sz, [_i, _i, _i]),

@@ -25,6 +25,10 @@ class DeltaConfig:
     sparse_factor: Fraction = field(default=Fraction(2, 1))
     # group size of the fp16 scales along the input dimension; -1 = one scale per output channel
     group_size: int = -1
+    # every delta layer keeps a second copy of its base weight in the tiled form the fused kernel
+    # streams fastest (calls of up to 128 tokens read it, larger ones the row-major weight); off:
+    # the base weight is held once and read row-major by every call
+    tile_base_weights: bool = True
 
     def __post_init__(self):
         if self.max_cpu_deltas is None:

@@ -103,6 +103,7 @@ struct MdlParams {
   int T, K, N, S, G, gs;
   int accumulate, ldy, nsplit, cb;
   int NP, NKB, NPG;
+  int base_tiled;    // wb holds the base weight in tiles (dz_layout.h) instead of row-major [N, K]
 };
 
 // Up to DZ_MAX_BATCH layer calls in one launch; np_end[j] = n-pairs of calls 0..j (entries beyond

@@ -420,6 +420,23 @@ __global__ __launch_bounds__(128) void dz_deal_kernel(const long long* __restric
   if (tid < T) perm_out[s_pos[leader] + rin] = tid;
 }
 
+// Base weight, row-major [N, K] -> tiles (dz_layout.h: dz_base_tile_offset / dz_base_frag_offset).
+// One thread moves 16 bytes: output chunk c = ((tile * 16 + fragment) * 64 + lane).
+__global__ __launch_bounds__(256) void dz_tile_base_kernel(const u4_t* __restrict__ w, u4_t* __restrict__ out,
+                                                           int K, int N) {
+  const long long c = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (c >= (long long)N * K / 8) return;
+  const int lane = (int)(c & 63), frag = (int)((c >> 6) & 15);
+  const long long tile = c >> 10;
+  const int nkb = K / DZ_KBLOCK;
+  const int np = (int)(tile / nkb), kb = (int)(tile % nkb);
+  const int h = frag & 1, j = (frag >> 1) & 3, s = frag >> 3;
+  const int i = lane & 15, g = lane >> 4;
+  const long long row = (long long)np * DZ_NPAIR + 16 * s + i;
+  const int col = kb * DZ_KBLOCK + 64 * j + 16 * g + 8 * h;
+  out[c] = w[(row * K + col) / 8];
+}
+
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
@@ -631,12 +648,12 @@ size_t dz_workspace_bytes(int T, int K, int N) {
   return WS_HEADER + WS_PERM_BYTES + (size_t)MAX_KSPLIT * 32 * (size_t)N * 4;
 }
 
-int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
-                                const void* const* codes_stacked, const void* const* meta_stacked,
-                                const void* const* scales_stacked, const int64_t* indices,
-                                uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
-                                int bits, int group_size, int accumulate, const int32_t* order,
-                                void* workspace, size_t workspace_bytes, void* stream) {
+static int multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
+                                    const void* const* codes_stacked, const void* const* meta_stacked,
+                                    const void* const* scales_stacked, const int64_t* indices,
+                                    uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
+                                    int bits, int group_size, int accumulate, const int32_t* order,
+                                    void* workspace, size_t workspace_bytes, void* stream, int base_tiled) {
   if (ncalls < 1 || ncalls > DZ_MAX_BATCH_CALLS) return DZ_ESHAPE;
   if (!x || !w_base || !indices || !y || !N || !ldy) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
@@ -687,6 +704,7 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
     Q.accumulate = accumulate; Q.ldy = ldy[j];
     Q.NP = N[j] / DZ_NPAIR; Q.NKB = K / DZ_KBLOCK;
     Q.nsplit = 1; Q.cb = Q.NKB; Q.NPG = 0;
+    Q.base_tiled = (base_tiled && w_base[j]) ? 1 : 0;
     Q.perm = T <= 32 ? nullptr : (order ? order : perm);
     Q.tok0 = 0;
     Q.nchunk = 1;
@@ -699,6 +717,37 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
   if (T > 32 && !order)
     hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
   return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override.load(std::memory_order_relaxed));
+}
+
+int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,
+                                const void* const* codes_stacked, const void* const* meta_stacked,
+                                const void* const* scales_stacked, const int64_t* indices,
+                                uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
+                                int bits, int group_size, int accumulate, const int32_t* order,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  return multi_delta_linear_batch(ncalls, x, w_base, codes_stacked, meta_stacked, scales_stacked, indices, y, N, ldy,
+                                  T, K, S, bits, group_size, accumulate, order, workspace, workspace_bytes, stream, 0);
+}
+
+int dz_multi_delta_linear_batch_tiled(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base_tiled,
+                                      const void* const* codes_stacked, const void* const* meta_stacked,
+                                      const void* const* scales_stacked, const int64_t* indices,
+                                      uint16_t* const* y, const int* N, const int* ldy, int T, int K, int S,
+                                      int bits, int group_size, int accumulate, const int32_t* order,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  return multi_delta_linear_batch(ncalls, x, w_base_tiled, codes_stacked, meta_stacked, scales_stacked, indices, y, N,
+                                  ldy, T, K, S, bits, group_size, accumulate, order, workspace, workspace_bytes,
+                                  stream, 1);
+}
+
+int dz_tile_base(const uint16_t* w, int K, int N, uint16_t* out, void* stream) {
+  if (!w || !out) return DZ_EINVAL;
+  if (K < DZ_KBLOCK || N < DZ_NPAIR || K % DZ_KBLOCK || N % DZ_NPAIR) return DZ_ESHAPE;
+  if (((uintptr_t)w & 15) || ((uintptr_t)out & 15)) return DZ_EALIGN;
+  const long long chunks = (long long)N * K / 8;   // 16 bytes each
+  hipLaunchKernelGGL(dz_tile_base_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const u4_t*)w, (u4_t*)out, K, N);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
 int dz_token_order(const int64_t* indices, int T, int S, int32_t* order, void* stream) {

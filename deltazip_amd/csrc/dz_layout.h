@@ -45,6 +45,14 @@ DZ_HD static inline size_t dz_code2_word(int np, int kb, int la, int j, int nkb)
 DZ_HD static inline size_t dz_code4_word(int np, int kb, int la, int j, int s, int nkb) {
   return ((((size_t)np * nkb + kb) * 2 + (j >> 1)) * 64 + la) * 4 + 2 * (j & 1) + s;
 }
+// Base weight in tiles (optional; the fused kernel for up to 128 tokens reads either form).  Tile
+// (np, kb) = 32 rows x 256 columns = 16 KiB, stored contiguously; inside it 16 fragments of 1 KiB,
+// fragment (s, j, h) = the dense operand of one v_mfma_f32_16x16x32_f16: lane la = 16*g + i holds
+// the 8 values W[32*np + 16*s + i][256*kb + 64*j + 16*g + 8*h + e], e = 0..7 (16 bytes per lane, a
+// wavefront reads one fragment per load).  The matching activation order is the one the kernel
+// uses for the row-major form, so both forms give the same sums in the same order.
+DZ_HD static inline size_t dz_base_tile_offset(int np, int kb, int nkb) { return ((size_t)np * nkb + kb) * 16384; }
+DZ_HD static inline int dz_base_frag_offset(int s, int j, int h) { return ((s * 4 + j) * 2 + h) * 1024; }
 DZ_HD static inline int dz_meta_shift(int s, int e) { return 16 * s + 2 * e; }
 DZ_HD static inline int dz_code2_shift(int s, int e) { return 2 * (4 * s + (e >> 1)) + 16 * (e & 1); }
 DZ_HD static inline int dz_code4_shift(int e) { return 4 * (e >> 1) + 16 * (e & 1); }

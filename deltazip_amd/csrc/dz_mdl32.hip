@@ -29,9 +29,11 @@ constexpr int WK32 = 4;
 constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is about a microsecond)
 
 // The work of one workgroup: n-pair `np`, K-slice `kc`, token chunk `ch` of the layer call P.
-template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY, bool IDL>
+template <int BITS, int TT, int PRE, int BASE, bool EARLY, bool IDL>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
+  constexpr bool HAS_BASE = BASE != 0;     // 1: base weight row-major [N, K]; 2: in tiles (dz_layout.h)
+  constexpr bool TILED = BASE == 2;
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? (PRE == 2 ? 3 : 4) : (TT == 2 ? 2 : 3);   // deltas per batch (two batches are in flight); 3 where 4 would not fit the registers
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
@@ -106,6 +108,20 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // bytes.  The matrix instruction wants row jj in lane jj, so before use the upper eight lanes of
   // each group of 16 trade places between the two halves (`base_operands`).
   auto issue_base = [&](int kb, int lane_r, const int s_lo, const int s_hi) {   // row fragments s_lo .. s_hi - 1
+    if constexpr (TILED) {
+      // the tile is 16 requests of 1 KiB, each already in the order the matrix instruction takes
+      const char* tb = (const char*)P.wb + dz_base_tile_offset(np, kb, P.NKB) + ((size_t)lane_r << 4);
+#pragma unroll
+      for (int s = s_lo; s < s_hi; ++s)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            const u4_t* q = (const u4_t*)(tb + dz_base_frag_offset(s, j, h));
+            a[s][j][h] = P.nchunk > 1 ? *q : __builtin_nontemporal_load(q);
+          }
+      return;
+    }
     const char* wbb = (const char*)(P.wb + (size_t)n0 * P.K + (size_t)kb * DZ_KBLOCK);
     const unsigned loff = (unsigned)(lane_r & 7) * Kb + (unsigned)(lane_r >> 4) * 32u + (unsigned)((lane_r >> 3) & 1) * 16u;
     // One chunk of tokens: the tile is read once in the whole launch and is requested as streaming
@@ -135,6 +151,11 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // jj >= 8 take it from lane jj - 8 of the second half's); v: row jj, chunk 2*ga + 1.
   auto base_operands = [&](const u4_t& ra, const u4_t& rb, h8_t& u, h8_t& v) {
     H8U uu, vv;
+    if constexpr (TILED) {
+      uu.v = ra; vv.v = rb;
+      u = uu.h; v = vv.h;
+      return;
+    }
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       // row_ror:8 inside each group of 16 lanes; bank mask 0xC = lanes 8..15, 0x3 = lanes 0..7
@@ -547,21 +568,21 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
 // that their partial sums can meet in that XCD's L2.  A launch may carry up to 4 chunks of 32 tokens
 // (33..128 tokens, grouped by delta id): the workgroups of the chunks of one (n-pair, k-chunk)
 // follow each other on the same XCD, so the base tile they all read comes from HBM once.
-template <int BITS, int TT, int PRE, bool HAS_BASE, bool EARLY>
+template <int BITS, int TT, int PRE, int BASE, bool EARLY>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_kernel(const MdlParams P) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
   const int per = P.nsplit * P.nchunk, rem = q % per;
   const int np = (q / per) * 8 + xcd, kc = rem / P.nchunk, ch = rem % P.nchunk;
   if (np >= P.NP) return;
-  mdl32_body<BITS, TT, PRE, HAS_BASE, EARLY, true>(P, np, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, BASE, EARLY, true>(P, np, kc, ch, smem);
 }
 
 // Several layer calls that share tokens, K and the slot table (the projections a fused layer
 // would hold in one weight: q/k/v, gate/up) in one launch: the n-pairs of the calls are numbered
 // through, a workgroup picks its call by its n-pair.  One call's tail (reduction, stores) then
 // overlaps the next one's loads instead of leaving the memory system idle between launches.
-template <int BITS, int TT, int PRE, bool HAS_BASE>
+template <int BITS, int TT, int PRE, int BASE>
 __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlBatch B) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
@@ -571,7 +592,7 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlB
   // wavefront-uniform choice among the calls (np_end of unused entries repeats the total)
   const int j = (npg >= B.np_end[0]) + (npg >= B.np_end[1]) + (npg >= B.np_end[2]);
   const int first = j == 0 ? 0 : B.np_end[j - 1];
-  mdl32_body<BITS, TT, PRE, HAS_BASE, false, false>(B.p[j], npg - first, kc, ch, smem);
+  mdl32_body<BITS, TT, PRE, BASE, false, false>(B.p[j], npg - first, kc, ch, smem);
 }
 
 // K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each
@@ -606,6 +627,7 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
       B.p[j].nsplit = nsplit;
       np_total += B.p[j].NP;
       if ((B.p[j].wb != nullptr) != has_base) return DZ_EINVAL;   // all with a base weight or none
+      if (B.p[j].base_tiled != B.p[0].base_tiled) return DZ_EINVAL; // ... and all in the same layout
     }
     B.np_end[j] = np_total;
   }
@@ -613,8 +635,10 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2 + WK32 * 512;   // activation slices + the token ids
   // single launches of at most one turn (two workgroups per CU) take the variant that requests half
   // the base tile before the ids are in
-  const bool early = nprob == 1 && has_base && grid <= 2 * dz_cu_count();
-  static std::atomic<unsigned long long> attr_done[15];
+  const bool tiled = has_base && B.p[0].base_tiled != 0;
+  // (with the base weight in tiles the early half measured slower, not faster)
+  const bool early = nprob == 1 && has_base && !tiled && grid <= 2 * dz_cu_count();
+  static std::atomic<unsigned long long> attr_done[21];
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
     if (!dz_lds_limit_once(attr_done[slot], f, (int)lds)) return DZ_ELAUNCH;
@@ -624,12 +648,16 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   };
   auto pick = [&](auto pre_c) -> int {
     constexpr int PRE_ = decltype(pre_c)::value;
-    const int s0 = 5 * PRE_;
-    if (nprob > 1) return has_base ? go(dz_mdl32_kernel<BITS, TT, PRE_, true, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0)
-                                   : go(dz_mdl32_kernel<BITS, TT, PRE_, false, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, false>, s0 + 1);
-    if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, false, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, false>, s0 + 2);
-    return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, true, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0 + 3)
-                 : go(dz_mdl32_kernel<BITS, TT, PRE_, true, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, true>, s0 + 4);
+    const int s0 = 7 * PRE_;
+    if (nprob > 1) {
+      if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0);
+      return tiled ? go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 1)
+                   : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 2);
+    }
+    if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0 + 3);
+    if (tiled) return go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 4);
+    return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 1, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 5)
+                 : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 6);
   };
   int rc = pre == 2 ? pick(std::integral_constant<int, 2>{}) : pre == 1 ? pick(std::integral_constant<int, 1>{})
                                                                        : pick(std::integral_constant<int, 0>{});

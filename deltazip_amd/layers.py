@@ -85,6 +85,7 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.qweight_stacked = torch.zeros((max_deltas,) + qs, dtype=torch.int32, device=w.device)
         self.meta_stacked = torch.zeros((max_deltas,) + ms, dtype=torch.int16, device=w.device)
         self.scales_stacked = torch.zeros((max_deltas,) + ss, dtype=torch.float16, device=w.device)
+        self.base_tiled = ops.tile_base(w.contiguous()) if delta_config.tile_base_weights and w.is_cuda else None
 
     def reset_delta(self, index: int):
         # all-zero scales make the slot contribute exactly 0 whatever the packed words hold
@@ -124,7 +125,7 @@ class LinearWithDelta(BaseLayerWithDelta):
         T = self.indices_len[0]
         order = self.token_order[:T] if self.token_order is not None and 32 < T <= ops.MAX_TOKENS_FUSED else None
         return ops.apply_delta(x, self.qweight_stacked, self.scales_stacked, self.meta_stacked,
-                               self.indices[:T], self.base_layer.weight, order=order)
+                               self.indices[:T], self.base_layer.weight, order=order, base_tiled=self.base_tiled)
 
     def forward(self, input_):
         skip_bias_add = getattr(self.base_layer, "skip_bias_add", False)

@@ -421,6 +421,26 @@ def _infer(qweight_stacked, scales_stacked, N: int):
     return S, words, G
 
 
+def tile_base(weight: torch.Tensor) -> torch.Tensor:
+    """The base weight [N, K] in the tiled form the fused kernel streams fastest (`dz_tile_base`):
+    a tensor of the same shape and dtype whose bytes are the tiles.  A layer converts its base
+    weight once and hands both forms to `multi_delta_linear` / `apply_delta_batch` (`base_tiled=`);
+    calls of up to 128 tokens read the tiles, larger ones the row-major weight."""
+    _need_cuda(weight)
+    if weight.dtype != torch.float16 or weight.dim() != 2 or not weight.is_contiguous():
+        raise ValueError("weight must be a contiguous float16 [N, K] tensor")
+    N, K = weight.shape
+    out = torch.empty_like(weight)
+    _lib.check(_lib.lib().dz_tile_base(weight.data_ptr(), K, N, out.data_ptr(), _stream()), "dz_tile_base")
+    return out
+
+
+def _check_tiled(base_tiled, base_weight) -> None:
+    if base_weight is None or base_tiled.shape != base_weight.shape or base_tiled.dtype != torch.float16 \
+            or not base_tiled.is_contiguous() or base_tiled.device != base_weight.device:
+        raise ValueError("base_tiled must be tile_base(base_weight)")
+
+
 def takes_fused_chunks(T: int, S: int) -> bool:
     """Whether a batch above the fused kernel's 128 tokens goes through it in chunks of 128 rather than
     through the matrix-core kernel.  That kernel works on row blocks of up to 256 tokens of one delta
@@ -435,10 +455,13 @@ def takes_fused_chunks(T: int, S: int) -> bool:
 def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qweight_stacked,
                        scales_stacked, meta_stacked, indices: torch.Tensor, *, bits: int,
                        out: Optional[torch.Tensor] = None, accumulate: bool = False,
-                       order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       order: Optional[torch.Tensor] = None,
+                       base_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ W_base^T + x @ dequant(delta[indices])^T.  `out` may be a column slice of a wider
     tensor (last-dim stride 1); with accumulate=True the result is added to it.  `order`: the
-    result of `token_order(indices, S)` when the caller already has it for this batch."""
+    result of `token_order(indices, S)` when the caller already has it for this batch.
+    `base_tiled`: `tile_base(base_weight)`, read instead of the row-major weight by calls of up to
+    128 tokens (the results are the same bit for bit)."""
     _need_cuda(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices)
     if x.dtype != torch.float16:
         raise ValueError("x must be float16")
@@ -480,13 +503,23 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
             for r in range(0, T, MAX_TOKENS_FUSED):
                 multi_delta_linear(x2[r:r + MAX_TOKENS_FUSED], base_weight, qweight_stacked, scales_stacked,
                                    meta_stacked, indices[r:r + MAX_TOKENS_FUSED], bits=bits,
-                                   out=out[r:r + MAX_TOKENS_FUSED], accumulate=accumulate)
+                                   out=out[r:r + MAX_TOKENS_FUSED], accumulate=accumulate, base_tiled=base_tiled)
             return out
         from .prefill import multi_delta_linear_prefill
         return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
                                           indices, bits=bits, out=out, accumulate=accumulate)
     ws = _workspace(x.device, T, K, N)
     optr = _order_ptr(order, T, x.device)
+    if base_tiled is not None:
+        _check_tiled(base_tiled, base_weight)
+        one = lambda p: (C.c_void_p * 1)(p)
+        rc = _lib.lib().dz_multi_delta_linear_batch_tiled(
+            1, one(x2.data_ptr()), one(base_tiled.data_ptr()), one(qweight_stacked.data_ptr()),
+            one(meta_stacked.data_ptr()), one(scales_stacked.data_ptr()), indices.data_ptr(), one(out.data_ptr()),
+            (C.c_int * 1)(N), (C.c_int * 1)(ldy), T, K, S, bits, group_size, 1 if accumulate else 0, optr,
+            ws.data_ptr(), ws.numel(), _stream())
+        _lib.check(rc, "dz_multi_delta_linear_batch_tiled")
+        return out
     if optr is None:
         rc = _lib.lib().dz_multi_delta_linear(
             x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
@@ -514,13 +547,14 @@ def _bits_from_shapes(qweight_stacked: torch.Tensor, K: int, N: int) -> int:
 
 def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: torch.Tensor,
                 meta_stacked: torch.Tensor, indices: torch.Tensor, base_weight: torch.Tensor,
-                order: Optional[torch.Tensor] = None) -> torch.Tensor:
+                order: Optional[torch.Tensor] = None, base_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Drop-in for serving/vllm/delta/deltazip_marlin.py:10-19.  Returns a new [T, N] tensor;
-    indices == -1 selects the base weight only.  (`order`: optional, see `token_order`.)"""
+    indices == -1 selects the base weight only.  (`order`: optional, see `token_order`; `base_tiled`:
+    optional, see `tile_base`.)"""
     N, K = base_weight.shape
     bits = _bits_from_shapes(qweight_stacked, K, N)
     y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits,
-                           order=order)
+                           order=order, base_tiled=base_tiled)
     return y.view(*x.shape[:-1], N)
 
 
@@ -535,7 +569,8 @@ def _order_ptr(order: Optional[torch.Tensor], T: int, device) -> Optional[int]:
 
 def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked: Sequence[torch.Tensor],
                       meta_stacked: Sequence[torch.Tensor], indices: torch.Tensor,
-                      base_weight: Sequence[torch.Tensor], order: Optional[torch.Tensor] = None):
+                      base_weight: Sequence[torch.Tensor], order: Optional[torch.Tensor] = None,
+                      base_tiled: Optional[Sequence[torch.Tensor]] = None):
     """`apply_delta` for up to 4 projections that share the tokens -- q/k/v or gate/up held as
     separate weights, which the reference fuses into one layer
     (serving/vllm/delta/layers_marlin.py:281-487) -- in one launch.  `x` is one [T, K] tensor for
@@ -551,7 +586,8 @@ def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked
     G = scales_stacked[0][0].numel() // base_weight[0].shape[0]
     S = qweight_stacked[0].shape[0]
     if T > MAX_TOKENS_FUSED:
-        return [apply_delta(xs[j], qweight_stacked[j], scales_stacked[j], meta_stacked[j], indices, base_weight[j])
+        return [apply_delta(xs[j], qweight_stacked[j], scales_stacked[j], meta_stacked[j], indices, base_weight[j],
+                            base_tiled=None if base_tiled is None else base_tiled[j])
                 for j in range(n)]
     _need_cuda(indices, *xs, *qweight_stacked, *scales_stacked, *meta_stacked, *base_weight)
     if indices.dtype != torch.int64 or indices.numel() != T or not indices.is_contiguous():
@@ -575,8 +611,15 @@ def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked
     vp = C.c_void_p * n
     ptrs = lambda ts: vp(*[t.data_ptr() for t in ts])
     ws = _workspace(x2s[0].device, T, K, sum(Ns))
-    rc = _lib.lib().dz_multi_delta_linear_batch(
-        n, ptrs(x2s), ptrs(base_weight), ptrs(qweight_stacked), ptrs(meta_stacked), ptrs(scales_stacked),
+    entry, bases = _lib.lib().dz_multi_delta_linear_batch, base_weight
+    if base_tiled is not None:
+        if len(base_tiled) != n:
+            raise ValueError("one tiled base weight per projection")
+        for j in range(n):
+            _check_tiled(base_tiled[j], base_weight[j])
+        entry, bases = _lib.lib().dz_multi_delta_linear_batch_tiled, base_tiled
+    rc = entry(
+        n, ptrs(x2s), ptrs(bases), ptrs(qweight_stacked), ptrs(meta_stacked), ptrs(scales_stacked),
         indices.data_ptr(), ptrs(outs), (C.c_int * n)(*Ns), (C.c_int * n)(*Ns), T, K, S, bits, group_size, 0,
         _order_ptr(order, T, indices.device), ws.data_ptr(), ws.numel(), _stream())
     _lib.check(rc, "dz_multi_delta_linear_batch")

@@ -232,6 +232,26 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
                                 int bits, int group_size, int accumulate, const int32_t* order,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
+/* The base weight in tiles.  The fused kernel reads a base weight 8 rows x 128 bytes per request
+ * from the row-major [N, K] form; from tiles -- 32 rows x 256 columns stored contiguously, in the
+ * order the matrix instruction takes its operand -- every request is 1 KiB of consecutive bytes,
+ * which the memory system streams faster.  A layer that keeps its base weight for the life of
+ * the model converts it once (as the deltas are repacked once): out has N*K elements like w.
+ * K % 256 == 0, N % 32 == 0.  No counterpart in the reference, whose base GEMM reads the
+ * parameter as it is (serving/vllm/delta/deltazip_marlin.py:10-19). */
+int dz_tile_base(const uint16_t* w, int K, int N, uint16_t* out, void* stream);
+
+/* dz_multi_delta_linear_batch with every w_base_tiled[j] in the tiled form dz_tile_base writes
+ * (ncalls = 1: the single layer call).  Same results, bit for bit, as with the row-major form. */
+int dz_multi_delta_linear_batch_tiled(int ncalls, const uint16_t* const* x,
+                                      const uint16_t* const* w_base_tiled,
+                                      const void* const* codes_stacked, const void* const* meta_stacked,
+                                      const void* const* scales_stacked, const int64_t* indices,
+                                      uint16_t* const* y, const int* N, const int* ldy, int T, int K,
+                                      int S, int bits, int group_size, int accumulate,
+                                      const int32_t* order, void* workspace, size_t workspace_bytes,
+                                      void* stream);
+
 /* The order in which the fused kernel takes the tokens of a batch of up to DZ_MAX_TOKENS_FUSED
  * tokens, 32 per chunk: order[T], a permutation of 0..T-1 in which the tokens of one delta stay
  * together and every chunk of 32 meets about the same number of distinct deltas.  Depends on the

@@ -297,6 +297,35 @@ def test_mid_size_batches_go_through_the_fused_kernel_in_chunks(dev, t, nd):
     assert np.abs(wide[:, 32:128].float().cpu().numpy() - dref).max() <= 2e-2 * np.abs(dref).max()
 
 
+@pytest.mark.parametrize("n,k,bits,gs,nd,t", [(64, 512, 2, -1, 3, 1), (96, 768, 4, 128, 5, 16), (256, 4096, 2, -1, 8, 32),
+                                              (160, 1024, 2, 64, 7, 33), (128, 2048, 4, -1, 12, 100), (512, 4096, 2, -1, 9, 128)])
+def test_tiled_base_weight_gives_the_same_bits(dev, n, k, bits, gs, nd, t):
+    """The base weight converted to tiles (dz_tile_base) feeds the fused kernel the same operands in the
+    same order: outputs equal the row-major call bit for bit, single and batched, and match the oracle.
+    The conversion itself is a pure rearrangement (every value kept, at the position dz_layout.h gives)."""
+    p = make_problem(n, k, bits, gs, nd, t, "uniform", 3000 + n + t, dev)
+    tiled = ops.tile_base(p["wb"])
+    w, tl = p["wb_np"], tiled.cpu().numpy().reshape(-1)
+    for (np_, kb, s_, j, h, lane) in [(0, 0, 0, 0, 0, 0), (n // 32 - 1, k // 256 - 1, 1, 3, 1, 63), (0, k // 256 - 1, 1, 2, 0, 37)]:
+        off = ((np_ * (k // 256) + kb) * 16384 + ((s_ * 4 + j) * 2 + h) * 1024 + lane * 16) // 2
+        i, g = lane % 16, lane // 16
+        row, col = 32 * np_ + 16 * s_ + i, 256 * kb + 64 * j + 16 * g + 8 * h
+        assert np.array_equal(tl[off:off + 8], w[row, col:col + 8])
+    assert np.array_equal(np.sort(tl.view(np.uint16)), np.sort(w.reshape(-1).view(np.uint16)))
+    y0 = run_layer(p)
+    y1 = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=tiled)
+    torch.cuda.synchronize()
+    assert torch.equal(y0, y1)
+    assert o.rel_err(y1.cpu().numpy(), o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])) <= TOL
+    b0 = ops.apply_delta_batch(p["x"], [p["q"]] * 2, [p["s"]] * 2, [p["m"]] * 2, p["ids"], [p["wb"]] * 2)
+    b1 = ops.apply_delta_batch(p["x"], [p["q"]] * 2, [p["s"]] * 2, [p["m"]] * 2, p["ids"], [p["wb"]] * 2,
+                               base_tiled=[tiled] * 2)
+    torch.cuda.synchronize()
+    assert torch.equal(b0[0], b1[0]) and torch.equal(b0[1], b1[1])
+    with pytest.raises(ValueError):
+        ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=tiled[:, : k // 2])
+
+
 def test_gemm_grouped(dev):
     """Grouped GEMM through the C ABI: ragged row blocks, a block without second weight, rows that no
     block covers (left untouched), an N that is not a multiple of the 256-wide tile, and the
