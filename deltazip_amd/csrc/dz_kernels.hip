@@ -744,6 +744,8 @@ int dz_tile_base(const uint16_t* w, int K, int N, uint16_t* out, void* stream) {
   if (!w || !out) return DZ_EINVAL;
   if (K < DZ_KBLOCK || N < DZ_NPAIR || K % DZ_KBLOCK || N % DZ_NPAIR) return DZ_ESHAPE;
   if (((uintptr_t)w & 15) || ((uintptr_t)out & 15)) return DZ_EALIGN;
+  const uintptr_t bytes = (uintptr_t)N * K * 2;
+  if ((uintptr_t)w < (uintptr_t)out + bytes && (uintptr_t)out < (uintptr_t)w + bytes) return DZ_EINVAL;   // a permutation: not in place
   const long long chunks = (long long)N * K / 8;   // 16 bytes each
   hipLaunchKernelGGL(dz_tile_base_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                      (const u4_t*)w, (u4_t*)out, K, N);

@@ -236,8 +236,8 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
  * from the row-major [N, K] form; from tiles -- 32 rows x 256 columns stored contiguously, in the
  * order the matrix instruction takes its operand -- every request is 1 KiB of consecutive bytes,
  * which the memory system streams faster.  A layer that keeps its base weight for the life of
- * the model converts it once (as the deltas are repacked once): out has N*K elements like w.
- * K % 256 == 0, N % 32 == 0.  No counterpart in the reference, whose base GEMM reads the
+ * the model converts it once (as the deltas are repacked once): out has N*K elements like w and
+ * must not overlap it (the conversion is a permutation).  K % 256 == 0, N % 32 == 0.  No counterpart in the reference, whose base GEMM reads the
  * parameter as it is (serving/vllm/delta/deltazip_marlin.py:10-19). */
 int dz_tile_base(const uint16_t* w, int K, int N, uint16_t* out, void* stream);
 

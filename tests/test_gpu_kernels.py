@@ -298,7 +298,8 @@ def test_mid_size_batches_go_through_the_fused_kernel_in_chunks(dev, t, nd):
 
 
 @pytest.mark.parametrize("n,k,bits,gs,nd,t", [(64, 512, 2, -1, 3, 1), (96, 768, 4, 128, 5, 16), (256, 4096, 2, -1, 8, 32),
-                                              (160, 1024, 2, 64, 7, 33), (128, 2048, 4, -1, 12, 100), (512, 4096, 2, -1, 9, 128)])
+                                              (160, 1024, 2, 64, 7, 33), (128, 2048, 4, -1, 12, 100), (512, 4096, 2, -1, 9, 128),
+                                              (256, 1024, 2, -1, 6, 200)])   # 200 tokens: two chunks through the fused kernel
 def test_tiled_base_weight_gives_the_same_bits(dev, n, k, bits, gs, nd, t):
     """The base weight converted to tiles (dz_tile_base) feeds the fused kernel the same operands in the
     same order: outputs equal the row-major call bit for bit, single and batched, and match the oracle.
@@ -324,6 +325,9 @@ def test_tiled_base_weight_gives_the_same_bits(dev, n, k, bits, gs, nd, t):
     assert torch.equal(b0[0], b1[0]) and torch.equal(b0[1], b1[1])
     with pytest.raises(ValueError):
         ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=tiled[:, : k // 2])
+    from deltazip_amd import _lib
+    assert _lib.lib().dz_tile_base(p["wb"].data_ptr(), k, n, p["wb"].data_ptr(), None) != 0      # not in place
+    assert _lib.lib().dz_tile_base(p["wb"].data_ptr(), k - 64, n, tiled.data_ptr(), None) != 0    # whole k-blocks only
 
 
 def test_gemm_grouped(dev):
