@@ -28,6 +28,7 @@ SIGNATURES = {
     "dz_multi_delta_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_compress_2of4": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dz_quant_scales": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp]),
+    "dz_quant_scales_mse": (_i, [_vp, _i, _i, _i, _i, C.c_float, _i, C.c_float, _vp, _vp, _vp]),
     "dz_pack_2of4": (_i, [_vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "dz_hessian_add": (_i, [_vp, _vp, _i, _i, _i, C.c_float, C.c_float, _vp]),
     "dz_obs_sweep": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),

@@ -263,6 +263,65 @@ __global__ __launch_bounds__(64) void dz_scales_kernel(const float* __restrict__
   }
 }
 
+// The same with the reference's grid search over the clipping range (deltazip/core/quant.py:85-101,
+// mse=True, sym): for i = 0 .. int(maxshrink * grid) - 1 the range is shrunk by p = 1 - i / grid,
+// the group is rounded to that grid and the candidate with the smallest sum of |q(x) - x|^norm
+// wins (the first one on a tie: `err < best`).  One wavefront per (row, scale group); the group
+// is re-read from cache for every candidate; sums: fp32 per lane in element order, then a
+// butterfly over the lanes.
+__global__ __launch_bounds__(64) void dz_scales_mse_kernel(const float* __restrict__ delta, int K, int N, int gs,
+                                                           int G, float maxq, float norm, int grid, int ncand,
+                                                           float* __restrict__ scale32,
+                                                           _Float16* __restrict__ scale16) {
+  const int row = blockIdx.x / G, g = blockIdx.x % G, lane = threadIdx.x;
+  const float* p = delta + (size_t)row * K + (size_t)g * gs;
+  float mn = 0.f, mx = 0.f;
+  for (int c = lane * 4; c < gs; c += 256) {
+    const f4_t v = *(const f4_t*)(p + c);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      mn = fminf(mn, v[e]);
+      mx = fmaxf(mx, v[e]);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o));
+    mx = fmaxf(mx, __shfl_xor(mx, o));
+  }
+  float xmin = mn, xmax = fmaxf(fabsf(mn), mx);
+  if (xmin < 0.f) xmin = -xmax;
+  if (xmin == 0.f && xmax == 0.f) {
+    xmin = -1.f;
+    xmax = 1.f;
+  }
+  const float zero = (maxq + 1.f) * 0.5f;
+  float best = INFINITY, best_scale = (xmax - xmin) / maxq;
+  for (int i = 0; i < ncand; ++i) {
+    const float pf = (float)(1.0 - (double)i / (double)grid);
+    const float sc = __fsub_rn(__fmul_rn(pf, xmax), __fmul_rn(pf, xmin)) / maxq;   // every product rounded, as the reference's tensor ops
+    float err = 0.f;
+    for (int c = lane * 4; c < gs; c += 256) {
+      const f4_t v = *(const f4_t*)(p + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float q = fminf(fmaxf(rintf(v[e] / sc) + zero, 0.f), maxq);
+        err += powf(fabsf(__fsub_rn(__fmul_rn(sc, q - zero), v[e])), norm);
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) err += __shfl_xor(err, o);
+    if (err < best) {
+      best = err;
+      best_scale = sc;
+    }
+  }
+  if (lane == 0) {
+    scale32[(size_t)g * N + row] = best_scale;
+    scale16[(size_t)g * N + row] = (_Float16)best_scale;
+  }
+}
+
 // One wavefront per (n-pair, k-block) tile; lane 16*ga + i produces its own four words of the
 // native arrays from rows i and 16 + i, columns 64*j + 16*ga .. + 15 of the k-block.
 //   pruning   in every aligned group of 4 columns the 2 values of largest magnitude stay (ties:
@@ -617,6 +676,22 @@ int dz_quant_scales(const float* delta, int K, int N, int bits, int group_size, 
   const int G = K / gs;
   hipLaunchKernelGGL(dz_scales_kernel, dim3((unsigned)N * G), dim3(64), 0, (hipStream_t)stream, delta, K, N, gs, G,
                      (float)((1 << bits) - 1), scale32, (_Float16*)scale16);
+  return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+int dz_quant_scales_mse(const float* delta, int K, int N, int bits, int group_size, float norm, int grid,
+                        float maxshrink, float* scale32, uint16_t* scale16, void* stream) {
+  if (!delta || !scale32 || !scale16) return DZ_EINVAL;
+  if (!(norm > 0.f) || grid < 1 || !(maxshrink >= 0.f) || maxshrink > 1.f) return DZ_EINVAL;
+  int rc = dz_native_sizes(K, N, bits, group_size, nullptr, nullptr, nullptr);
+  if (rc) return rc;
+  int gs;
+  if ((rc = check_group(K, group_size, &gs))) return rc;
+  if ((uintptr_t)delta & 15) return DZ_EALIGN;
+  const int G = K / gs;
+  const int ncand = (int)((double)maxshrink * (double)grid);   // int(maxshrink * grid), quant.py:87
+  hipLaunchKernelGGL(dz_scales_mse_kernel, dim3((unsigned)N * G), dim3(64), 0, (hipStream_t)stream, delta, K, N, gs,
+                     G, (float)((1 << bits) - 1), norm, grid, ncand, scale32, (_Float16*)scale16);
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 

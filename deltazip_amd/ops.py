@@ -257,9 +257,12 @@ def compress_delta(delta: torch.Tensor, bits: int, group_size: int = -1):
     return q, m, s
 
 
-def quant_scales(delta: torch.Tensor, bits: int, group_size: int = -1):
+def quant_scales(delta: torch.Tensor, bits: int, group_size: int = -1, mse: bool = False, norm: float = 2.4,
+                 grid: int = 100, maxshrink: float = 0.8):
     """Symmetric scales of the reference's Quantizer.find_params (deltazip/core/quant.py:48-130,
-    perchannel, sym) for an fp32 delta [N, K] on the GPU: (scale32 [G, N] fp32, scale16 [G, N] fp16)."""
+    perchannel, sym) for an fp32 delta [N, K] on the GPU: (scale32 [G, N] fp32, scale16 [G, N] fp16).
+    mse=True runs the reference's search over the clipping range (quant.py:85-101) with its
+    `norm`, `grid` and `maxshrink`."""
     _need_cuda(delta)
     if delta.dtype != torch.float32 or delta.dim() != 2 or not delta.is_contiguous():
         raise ValueError("delta must be a contiguous float32 [N, K] tensor")
@@ -267,8 +270,13 @@ def quant_scales(delta: torch.Tensor, bits: int, group_size: int = -1):
     _, _, ss = stacked_shapes(K, N, bits, group_size)
     s32 = torch.empty(ss, dtype=torch.float32, device=delta.device)
     s16 = torch.empty(ss, dtype=torch.float16, device=delta.device)
-    rc = _lib.lib().dz_quant_scales(delta.data_ptr(), K, N, bits, group_size, s32.data_ptr(), s16.data_ptr(), _stream())
-    _lib.check(rc, "dz_quant_scales")
+    if mse:
+        rc = _lib.lib().dz_quant_scales_mse(delta.data_ptr(), K, N, bits, group_size, float(norm), int(grid),
+                                            float(maxshrink), s32.data_ptr(), s16.data_ptr(), _stream())
+        _lib.check(rc, "dz_quant_scales_mse")
+    else:
+        rc = _lib.lib().dz_quant_scales(delta.data_ptr(), K, N, bits, group_size, s32.data_ptr(), s16.data_ptr(), _stream())
+        _lib.check(rc, "dz_quant_scales")
     return s32, s16
 
 

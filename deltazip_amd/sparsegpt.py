@@ -20,8 +20,9 @@ from . import ops
 
 
 class Quantizer:
-    """Symmetric per-output-row weight quantizer (deltazip/core/quant.py:21-144 with the settings
-    deltazip/modeling/_base.py:399-406 uses: perchannel=True, sym=True, mse=False)."""
+    """Symmetric per-output-row weight quantizer (deltazip/core/quant.py:21-144; the settings
+    deltazip/modeling/_base.py:399-406 uses are perchannel=True, sym=True, mse=False; mse=True, the
+    search over the clipping range with `norm`, `grid` and `maxshrink`, is built too)."""
 
     def __init__(self):
         self.maxq = 0
@@ -29,18 +30,20 @@ class Quantizer:
         self.scale: Optional[torch.Tensor] = None
         self.zero: Optional[torch.Tensor] = None
 
-    def configure(self, bits, perchannel=True, sym=True, mse=False, **_):
+    def configure(self, bits, perchannel=True, sym=True, mse=False, norm=2.4, grid=100, maxshrink=0.8, grouprows=1):
         if bits not in (2, 4):
             raise NotImplementedError("Only 2 and 4 bits are supported.")
-        if not (perchannel and sym) or mse:
-            raise NotImplementedError("only the per-channel symmetric quantizer without MSE search is built")
+        if not (perchannel and sym) or grouprows != 1:
+            raise NotImplementedError("only the per-channel symmetric quantizer is built")
         self.bits = bits
         self.maxq = 2 ** bits - 1
+        self.mse, self.norm, self.grid, self.maxshrink = bool(mse), norm, grid, maxshrink
 
     def find_params(self, x: torch.Tensor, weight: bool = True):
         if not weight:
             raise NotImplementedError("activation quantisation is not part of this path")
-        s32, _ = ops.quant_scales(x.float().contiguous(), self.bits, -1)
+        s32, _ = ops.quant_scales(x.float().contiguous(), self.bits, -1, mse=self.mse, norm=self.norm, grid=self.grid,
+                                  maxshrink=self.maxshrink)
         self.scale = s32.reshape(-1, 1)                                  # [N, 1], as quant.py:118-121
         self.zero = torch.full_like(self.scale, (self.maxq + 1) / 2)
 

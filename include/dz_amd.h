@@ -148,6 +148,14 @@ int dz_quant_scales(const float* delta, int K, int N, int bits, int group_size, 
 int dz_pack_2of4(const float* w, const float* scale32, int K, int N, int bits, int group_size, void* out_codes,
                  void* out_meta, void* stream);
 
+/* dz_quant_scales with the search over the clipping range that Quantizer.find_params runs for
+ * mse=True (deltazip/core/quant.py:85-101; sym, perchannel): for i = 0 .. int(maxshrink * grid) - 1
+ * the symmetric range is shrunk by p = 1 - i / grid and the candidate whose rounding error
+ * sum |q(x) - x|^norm over the row (or scale group) is smallest gives the scale; the first
+ * candidate wins a tie.  The reference's defaults are norm = 2.4, grid = 100, maxshrink = 0.8. */
+int dz_quant_scales_mse(const float* delta, int K, int N, int bits, int group_size, float norm, int grid,
+                        float maxshrink, float* scale32, uint16_t* scale16, void* stream);
+
 /* Layer Hessian of SparseGPT.add_batch (deltazip/core/sparsegpt.py:27-40):
  * H <- H * scale_h + (scale_x * x)^T (scale_x * x) for x [T, K] (fp16 if x_is_fp16, else fp32),
  * H [K, K] fp32; the caller passes scale_h = n / (n + b) and scale_x = sqrt(2 / (n + b)) for b new

@@ -9,6 +9,9 @@ Every function names the reference lines it follows (paths relative to the refer
 
 Pinning status (what independent evidence each function is checked against in tests/):
   quantize, find_params_sym     closed forms + known answers computed by hand          (pinned)
+  find_params_sym(mse=True)     every candidate's error against plain-Python loops on exactly
+                                representable rows, first-minimum rule, invariants      (pinned; the
+                                reference's torch.sum order is undefined: near-ties may differ)
   prune_2of4_magnitude          brute force on tiny rows, group invariants             (pinned)
   pack_gptq / unpack_gptq       single-bit probes, hand-packed words, round trips      (pinned)
   dequant_gptq                  exhaustive fp16-scale sweep against exact rational math (pinned)
@@ -52,11 +55,13 @@ def quantize_codes(x, scale, zero, maxq):
     return np.clip(np.rint(x / scale) + zero, 0, maxq).astype(np.uint8)
 
 
-def find_params_sym(w: np.ndarray, bits: int, group_size: int = -1):
+def find_params_sym(w: np.ndarray, bits: int, group_size: int = -1, mse: bool = False, norm: float = 2.4,
+                    grid: int = 100, maxshrink: float = 0.8, return_errors: bool = False):
     """Symmetric per-output-row (optionally per (row, K-group)) scale and zero.
 
-    deltazip/core/quant.py:48-130 with perchannel=True, sym=True, mse=False, weight=True
-    (the configuration deltazip/modeling/_base.py:399-406 uses).  `w` is [N, K] fp32.
+    deltazip/core/quant.py:48-130 with perchannel=True, sym=True, weight=True; mse=False is the
+    configuration deltazip/modeling/_base.py:399-406 uses, mse=True adds the search over the
+    clipping range (`_mse_search`).  `w` is [N, K] fp32.
     Returns (scale [N, G] fp32, zero [N, G] fp32) with G = 1 for group_size == -1.
 
     The reference computes the parameters on the un-pruned delta (core/sparsegpt.py:64-66).
@@ -79,7 +84,39 @@ def find_params_sym(w: np.ndarray, bits: int, group_size: int = -1):
     xmax = np.where(both0, +1.0, xmax).astype(np.float32)
     scale = ((xmax - xmin) / np.float32(maxq)).astype(np.float32)   # quant.py:81
     zero = np.full_like(scale, (maxq + 1) / 2)                      # quant.py:83
+    if mse:
+        scale, errs = _mse_search(wg, xmin, xmax, scale, zero, maxq, norm, grid, maxshrink)
+        if return_errors:
+            return scale, zero, errs
     return scale, zero
+
+
+def _mse_search(wg, xmin, xmax, scale, zero, maxq, norm, grid, maxshrink):
+    """deltazip/core/quant.py:85-101 for sym=True: candidates p = 1 - i / grid, i = 0 ..
+    int(maxshrink * grid) - 1; every candidate's range is (p * xmin, p * xmax), its scale
+    (xmax1 - xmin1) / maxq, its zero the symmetric one; the error of a row (group) is the sum of
+    |quantize(x) - x| ** norm, and a candidate replaces the best so far only when strictly better
+    (`err < best`).  The elementwise arithmetic is fp32 as the reference's tensor ops; the
+    reference's torch.sum has no defined order, here the sum is taken in float64.  Returns the
+    chosen scale and the errors of all candidates [ncand, N, G] (for tests of near-ties)."""
+    scale = scale.copy()
+    best = np.full(scale.shape, np.inf)
+    ncand = int(maxshrink * grid)
+    errs = np.empty((ncand,) + scale.shape)
+    for i in range(ncand):
+        p = np.float32(1 - i / grid)                                 # a Python float times an fp32 tensor
+        xmin1 = (p * xmin).astype(np.float32)
+        xmax1 = (p * xmax).astype(np.float32)
+        scale1 = ((xmax1 - xmin1) / np.float32(maxq)).astype(np.float32)
+        q = quantize(wg, scale1[:, :, None], zero[:, :, None], maxq)   # quant.py:93
+        d = np.abs((q - wg).astype(np.float32))
+        e = np.power(d, np.float32(norm), dtype=np.float32)
+        err = e.astype(np.float64).sum(axis=2)
+        errs[i] = err
+        better = err < best
+        best = np.where(better, err, best)
+        scale = np.where(better, scale1, scale).astype(np.float32)
+    return scale, errs
 
 
 # --------------------------------------------------------------------------------------

@@ -84,6 +84,9 @@ def test_compressor_entry_points_check_their_arguments(dzlib):
     assert sweep(pn=2, pm=16) == -2
     assert dzlib.dz_quant_scales(one, 256, 32, 3, -1, one, one, None) == -3
     assert dzlib.dz_quant_scales(one, 256, 32, 4, 100, one, one, None) == -4
+    assert dzlib.dz_quant_scales_mse(one, 256, 32, 3, -1, 2.4, 100, 0.8, one, one, None) == -3
+    assert dzlib.dz_quant_scales_mse(one, 256, 32, 4, -1, 2.4, 0, 0.8, one, one, None) == -1      # grid >= 1
+    assert dzlib.dz_quant_scales_mse(one, 256, 32, 4, -1, 2.4, 100, 1.5, one, one, None) == -1    # maxshrink in [0, 1]
     assert dzlib.dz_pack_2of4(one, None, 256, 32, 4, -1, one, one, None) == -1
     assert dzlib.dz_pack_2of4(one, one, 250, 32, 4, -1, one, one, None) == -2
 

@@ -56,6 +56,39 @@ def test_obs_sweep_bit_exact(dev, n, k, bits, quant, prune):
     assert np.array_equal(loss.cpu().numpy(), want_loss)
 
 
+@pytest.mark.parametrize("n,k,bits,gs", [(64, 512, 4, -1), (96, 1024, 2, -1), (32, 512, 4, 128), (64, 256, 2, 64)])
+def test_scales_with_the_search_over_the_clipping_range(dev, n, k, bits, gs):
+    """dz_quant_scales_mse against the oracle's restatement of quant.py:85-101.  The candidates'
+    errors are sums of |d| ** 2.4 whose last bits depend on the pow routine and the order of the
+    sum, so where two candidates are within 1e-5 of each other either may win; everywhere else the
+    chosen scale is the oracle's, bit for bit."""
+    W, _ = _inputs(n, k, 8, 40 + n + bits)
+    W[3, 5] = 25 * np.abs(W).max()                                # a row with an outlier
+    W[7] = 0                                                      # an all-zero row
+    W[9] = np.abs(W[9])                                           # a row without a negative value
+    s32, s16 = ops.quant_scales(torch.from_numpy(W).to(dev), bits, gs, mse=True)
+    scale, _, errs = o.find_params_sym(W, bits, gs, mse=True, return_errors=True)      # [N, G], [80, N, G]
+    plain, _ = o.find_params_sym(W, bits, gs)
+    got = s32.cpu().numpy().T                                                            # [N, G]
+    assert got.shape == scale.shape
+    differ = got != scale
+    assert differ.mean() < 0.05
+    for r, g in zip(*np.nonzero(differ)):
+        cand = np.array([np.float32(np.float32(1 - i / 100) * plain[r, g]) for i in range(80)])
+        i_got = int(np.argmin(np.abs(cand - got[r, g])))
+        assert abs(cand[i_got] - got[r, g]) <= 1e-6 * got[r, g]                          # one of the candidates ...
+        assert errs[i_got, r, g] <= errs[:, r, g].min() * (1 + 1e-5)                     # ... and as good as the best
+    assert (got <= plain).all() and (got < plain).any()           # the search only ever shrinks the range
+    assert np.array_equal(s16.cpu().numpy().view(np.uint16), s32.cpu().numpy().astype(np.float16).view(np.uint16))
+    # the Quantizer front end with the reference's keywords
+    from deltazip_amd.sparsegpt import Quantizer
+    qz = Quantizer()
+    qz.configure(bits, perchannel=True, sym=True, mse=True, norm=2.4, grid=100, maxshrink=0.8)
+    qz.find_params(torch.from_numpy(W).to(dev), weight=True)
+    if gs == -1:
+        assert torch.equal(qz.scale[:, 0], s32[0]) and float(qz.zero[0, 0]) == 2 ** (bits - 1)
+
+
 def test_scales_and_pack_match_the_reference_pipeline(dev):
     """Values on the grid with two zeros per group of four -> the same native bytes as compressing
     and packing the reference's way (oracle) and converting with the repacker."""

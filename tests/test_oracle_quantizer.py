@@ -107,3 +107,74 @@ def test_compress_delta_known_answers():
     assert keep.tolist() == [[True, True, False, False, True, False, True, False]]
     # scale = 0.008 / 15; 0.004 / scale = 7.5 -> 8 -> 16 -> 15; 0.001 / scale = 1.875 -> 2 -> 10
     assert codes.T.tolist() == [[15, 15, 8, 8, 8, 8, 10, 8]]
+
+
+# ---- the search over the clipping range (quant.py:85-101, mse=True) --------------------------------
+def _brute_force_mse(row, bits, norm, grid, maxshrink):
+    """Plain Python floats and loops: every candidate's error, the first minimum wins."""
+    import math
+    maxq, zero = 2 ** bits - 1, 2 ** (bits - 1)
+    xmin, xmax = min(min(row), 0.0), max(max(row), 0.0)
+    xmax = max(abs(xmin), xmax)
+    if xmin < 0:
+        xmin = -xmax
+    if xmin == 0 and xmax == 0:
+        xmin, xmax = -1.0, 1.0
+    out = []
+    for i in range(int(maxshrink * grid)):
+        p = 1 - i / grid
+        s = (p * xmax - p * xmin) / maxq
+        err = 0.0
+        for v in row:
+            # round half to even, as torch.round
+            q = min(max(round(v / s) + zero, 0), maxq)
+            err += abs(s * (q - zero) - v) ** norm
+        out.append((err, s))
+    return out
+
+
+@pytest.mark.parametrize("bits", [2, 4])
+def test_mse_search_against_brute_force(bits):
+    rng = np.random.default_rng(7 + bits)
+    for trial in range(40):
+        # multiples of 1/64 in [-2, 2]: exact in fp32, so float64 loops and the fp32 oracle see the same values
+        row = (rng.integers(-128, 129, size=12) / 64.0).astype(np.float32)
+        if trial % 5 == 0:
+            row[0] = 4.0                                              # an outlier: shrinking the range pays
+        scale, zero, errs = o.find_params_sym(row[None, :], bits, mse=True, return_errors=True)
+        cand = _brute_force_mse([float(v) for v in row], bits, 2.4, 100, 0.8)
+        assert errs.shape[0] == len(cand) == 80
+        np.testing.assert_allclose(errs[:, 0, 0], [c[0] for c in cand], rtol=2e-5, atol=1e-12)
+        best = min(c[0] for c in cand)
+        first = next(c for c in cand if c[0] == best)
+        chosen = float(scale[0, 0])
+        if abs(chosen - first[1]) > 1e-6 * first[1]:                  # only a near-tie may resolve differently
+            e_chosen = next(c[0] for c in cand if abs(c[1] - chosen) <= 1e-6 * c[1])
+            assert e_chosen <= best * (1 + 1e-5)
+        assert zero[0, 0] == 2 ** (bits - 1)
+
+
+def test_mse_search_with_only_the_full_range_as_candidate_changes_nothing():
+    rng = np.random.default_rng(3)
+    w = rng.standard_normal((5, 64)).astype(np.float32)
+    plain, _ = o.find_params_sym(w, 4)
+    one, _ = o.find_params_sym(w, 4, mse=True, grid=1, maxshrink=1.0)      # i = 0 only: p = 1
+    none, _ = o.find_params_sym(w, 4, mse=True, grid=100, maxshrink=0.0)   # no candidate at all
+    assert np.array_equal(plain, one) and np.array_equal(plain, none)
+
+
+def test_mse_search_shrinks_for_an_outlier_and_scales_with_the_row():
+    row = np.array([[1.0] + [0.3] * 20 + [-0.3] * 3], dtype=np.float32)
+    plain, _ = o.find_params_sym(row, 2)
+    searched, _, errs = o.find_params_sym(row, 2, mse=True, return_errors=True)
+    assert searched[0, 0] < plain[0, 0]
+    assert errs[:, 0, 0].min() < errs[0, 0, 0]                        # candidate 0 is the plain range
+    # the grid is relative to the row's range: a row twice as large gets exactly twice the scale
+    twice, _ = o.find_params_sym(2 * row, 2, mse=True)
+    assert twice[0, 0] == 2 * searched[0, 0]
+    # per group: each group is searched on its own
+    two = np.concatenate([row, 4 * row], axis=1)
+    two = np.pad(two, ((0, 0), (0, 128 - two.shape[1])))[:, :128]
+    g, _ = o.find_params_sym(np.concatenate([np.pad(row, ((0, 0), (0, 40))), np.pad(4 * row, ((0, 0), (0, 40)))], axis=1), 2,
+                             group_size=64, mse=True)
+    assert g.shape == (1, 2) and g[0, 0] == searched[0, 0] and g[0, 1] == 4 * searched[0, 0]
