@@ -1,7 +1,7 @@
 """Seeded random sweeps of the layer call against the oracle: shapes, bit widths, scale groupings,
 token counts on both sides of every internal threshold (16, 32, 128 tokens), id patterns with and
 without base-only tokens, and the ways a call can be made (plain, delta-only accumulate, into a
-column slice, batched).  Some kernel variants -- 2-bit deltas with scale groups of 64 in a batched
+column slice, batched; each with the base weight row-major and in tiles).  Some kernel variants -- 2-bit deltas with scale groups of 64 in a batched
 launch is the one under the highest register pressure -- are reached only by such combinations."""
 import numpy as np
 import pytest
@@ -35,8 +35,10 @@ def _check(dev, rng, n, k, bits, gs, nd, t, mode):
     p = make_problem(n, k, bits, gs, nd, t, ids, seed, dev)
     ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
     tol = TOL
+    tiled = ops.tile_base(p["wb"])   # every call with a base weight is made in both forms: same bits
     if mode == 0:
         y = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"])
+        assert torch.equal(y, ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=tiled)), case
     elif mode == 1:   # delta only, added to the base product (which is rounded to fp16 first)
         base16 = (p["x_np"].astype(np.float32) @ p["wb_np"].astype(np.float32).T).astype(np.float16)
         y = torch.from_numpy(base16).to(dev)
@@ -47,8 +49,15 @@ def _check(dev, rng, n, k, bits, gs, nd, t, mode):
         ops.multi_delta_linear(p["x"], p["wb"], p["q"], p["s"], p["m"], p["ids"], bits=bits, out=wide[:, 32:32 + n])
         assert float(wide[:, :32].abs().max()) == 0 and float(wide[:, 32 + n:].abs().max()) == 0, case
         y = wide[:, 32:32 + n]
+        wide2 = torch.zeros_like(wide)
+        ops.multi_delta_linear(p["x"], p["wb"], p["q"], p["s"], p["m"], p["ids"], bits=bits, out=wide2[:, 32:32 + n],
+                               base_tiled=tiled)
+        assert torch.equal(wide, wide2), case
     else:             # two calls in one launch
         y = ops.apply_delta_batch(p["x"], [p["q"]] * 2, [p["s"]] * 2, [p["m"]] * 2, p["ids"], [p["wb"]] * 2)[1]
+        yt = ops.apply_delta_batch(p["x"], [p["q"]] * 2, [p["s"]] * 2, [p["m"]] * 2, p["ids"], [p["wb"]] * 2,
+                                   base_tiled=[tiled] * 2)
+        assert torch.equal(y, yt[1]) and torch.equal(yt[0], yt[1]), case
     torch.cuda.synchronize()
     err = o.rel_err(y.float().cpu().numpy(), ref)
     assert err <= tol, (case, err)
