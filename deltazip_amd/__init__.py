@@ -15,7 +15,7 @@ from .layers import (BaseLayerWithDelta, ColumnParallelLinearWithDelta, DeltaMap
                      from_layer_logits_processor)
 from .manager import DeltaModelManager, LRUCacheDeltaModelManager, create_delta_manager
 from .ops import (add_delta, add_delta_slice, apply_delta, apply_delta_batch, apply_delta_into, apply_delta_packed_nslice, apply_delta_embed, apply_delta_uncompressed, compress_delta, dequant, merge, multi_delta_linear,
-                  native_sizes, repack_gptq_to_native, unrepack_native_to_gptq, segment, stacked_shapes, token_order)
+                  native_sizes, repack_gptq_to_native, unrepack_native_to_gptq, segment, stacked_shapes, tile_base, token_order)
 from .quant_linear import QuantLinear
 from .sparsegpt import Quantizer, SparseGPT
 
@@ -28,5 +28,5 @@ __all__ = [
     "DeltaLayerWeights", "DeltaModel", "convert_model", "compress_model", "save_compressed", "save_converted", "DeltaModelManager", "LRUCacheDeltaModelManager",
     "create_delta_manager", "LogitsProcessorWithDelta", "VocabParallelEmbeddingWithDelta",
     "from_layer_logits_processor", "apply_delta_embed", "apply_delta_uncompressed", "compress_delta", "apply_delta_batch", "token_order", "apply_delta_into", "apply_delta_packed_nslice",
-    "Quantizer", "SparseGPT", "lossy_compress",
+    "Quantizer", "SparseGPT", "lossy_compress", "tile_base",
 ]
