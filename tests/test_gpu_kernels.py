@@ -351,6 +351,48 @@ def test_tiled_base_weight_wide_launch_stays_unsplit(dev):
     assert torch.equal(y2, y3) and torch.equal(y3, y0)
 
 
+def test_fused_layer_calls_replay_from_a_graph(dev):
+    """What a serving loop does with a decode step: the layer calls -- a single projection over the
+    tiled base weight, two projections in one launch at 64 tokens (token order computed inside the
+    call), a split-K launch -- are captured once into a HIP graph and replayed after the ids were
+    rewritten in place, with eager work and synchronisations between the replays.  Every replay
+    equals the eager call bit for bit: nothing in the path reads back to the host, allocates or
+    depends on state a replay would find changed (the split-K workspace is left empty by every launch)."""
+    a = make_problem(256, 4096, 2, -1, 6, 24, "uniform", 501, dev)      # split in K
+    b = make_problem(160, 1024, 4, 128, 9, 64, "uniform", 502, dev)     # two chunks of tokens, grouped scales
+    tiled = ops.tile_base(a["wb"])
+
+    def step():
+        y0 = ops.apply_delta(a["x"], a["q"], a["s"], a["m"], a["ids"], a["wb"], base_tiled=tiled)
+        y1 = ops.apply_delta_batch(b["x"], [b["q"]] * 2, [b["s"]] * 2, [b["m"]] * 2, b["ids"], [b["wb"]] * 2)
+        return y0, y1[0], y1[1]
+
+    step()                                                               # one-time set-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            outs = step()
+    torch.cuda.current_stream().wait_stream(side)
+    rng = np.random.default_rng(5)
+    for rep in range(4):
+        ia, ib = rng.integers(-1, 6, size=24), rng.integers(-1, 9, size=64)
+        if rep == 2:
+            ia[:], ib[:] = -1, 3                                         # base only / one delta for every token
+        a["ids"].copy_(torch.from_numpy(ia).to(dev))
+        b["ids"].copy_(torch.from_numpy(ib).to(dev))
+        eager = step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(outs, eager):
+            assert torch.equal(got, want), rep
+        assert o.rel_err(outs[0].cpu().numpy(), o.forward_ref(a["x_np"], a["wb_np"], a["dts"], ia)) <= TOL
+        assert o.rel_err(outs[2].cpu().numpy(), o.forward_ref(b["x_np"], b["wb_np"], b["dts"], ib)) <= TOL
+
+
 def test_gemm_grouped(dev):
     """Grouped GEMM through the C ABI: ragged row blocks, a block without second weight, rows that no
     block covers (left untouched), an N that is not a multiple of the 256-wide tile, and the
