@@ -32,8 +32,16 @@ constexpr int DZ_SPIN_LIMIT = 1 << 16;   // polls of the partial sums (a poll is
 template <int BITS, int TT, int PRE, int BASE, bool EARLY, bool IDL>
 __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, const int kc, const int ch,
                                            unsigned char* smem) {
-  constexpr bool HAS_BASE = BASE != 0;     // 1: base weight row-major [N, K]; 2: in tiles (dz_layout.h)
-  constexpr bool TILED = BASE == 2;
+  // BASE: 0 no base weight; 1 row-major [N, K]; 2 in tiles (dz_layout.h); 3, 4 and 5: 1, 2 and 0
+  // for launches with several chunks of tokens (33 .. 128 tokens), where rows of x / idx / y go
+  // through the token order P.perm and the base tile is requested as cacheable data.  A
+  // compile-time choice: a wavefront-uniform branch around requests costs 3 % of the 7B step (the
+  // compiler's wait-count pass sees two paths with different requests outstanding and makes
+  // every later wait stricter).
+  constexpr bool HAS_BASE = BASE >= 1 && BASE <= 4;
+  constexpr bool TILED = BASE == 2 || BASE == 4;
+  constexpr bool MULTI = BASE >= 3;          // P.nchunk > 1 and P.perm != nullptr
+  constexpr bool SHARED_TILE = MULTI;
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? (PRE == 2 ? 3 : 4) : (TT == 2 ? 2 : 3);   // deltas per batch (two batches are in flight); 3 where 4 would not fit the registers
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
@@ -80,7 +88,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   auto issue_x = [&](int kb, int lane_r) {
     const char* xb = (const char*)(P.x + (size_t)kb * DZ_KBLOCK);
     const int c = lane_r & 31;
-    if (P.perm) {
+    if constexpr (MULTI) {
 #pragma unroll
       for (int i = 0; i < NX; ++i) {
         const int t = min(2 * i + (lane_r >> 5), Tc - 1);
@@ -118,7 +126,8 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
 #pragma unroll
           for (int h = 0; h < 2; ++h) {
             const u4_t* q = (const u4_t*)(tb + dz_base_frag_offset(s, j, h));
-            a[s][j][h] = P.nchunk > 1 ? *q : __builtin_nontemporal_load(q);
+            if constexpr (SHARED_TILE) a[s][j][h] = *q;
+            else a[s][j][h] = __builtin_nontemporal_load(q);
           }
       return;
     }
@@ -129,23 +138,16 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // too, a moment later, on the same XCD; an ordinary request leaves it in that L2 for them
     // (measured on 64 tokens / 4-bit deltas: 24 % more bytes from memory than the layer holds
     // when every chunk streams the tile for itself).
-    if (P.nchunk > 1) {
 #pragma unroll
-      for (int s = s_lo; s < s_hi; ++s)
+    for (int s = s_lo; s < s_hi; ++s)
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
-            a[s][j][h] = *(const u4_t*)(wbb + (size_t)(16 * s + 8 * h) * Kb + loff + 128 * j);
-    } else {
-#pragma unroll
-      for (int s = s_lo; s < s_hi; ++s)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int h = 0; h < 2; ++h)
-            a[s][j][h] = __builtin_nontemporal_load((const u4_t*)(wbb + (size_t)(16 * s + 8 * h) * Kb + loff + 128 * j));
-    }
+        for (int h = 0; h < 2; ++h) {
+          const u4_t* q = (const u4_t*)(wbb + (size_t)(16 * s + 8 * h) * Kb + loff + 128 * j);
+          if constexpr (SHARED_TILE) a[s][j][h] = *q;
+          else a[s][j][h] = __builtin_nontemporal_load(q);
+        }
   };
   // u: row jj, chunk 2*ga of step j (lanes jj < 8 have it in the first half's register, lanes
   // jj >= 8 take it from lane jj - 8 of the second half's); v: row jj, chunk 2*ga + 1.
@@ -192,7 +194,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     const unsigned id_lds = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem +
                             (unsigned)(WK32 * TP * DZ_KBLOCK * 2 + wave * 512);
     if (lane < Tc) {
-      prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
+      prow = MULTI ? P.perm[tok0 + lane] : tok0 + lane;
       const char* ip = (const char*)(P.idx + prow);
       asm volatile(
           "s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %2, off\n\t"
@@ -226,7 +228,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // ids return behind the activations, which are L2 hits and long in by then.
     const char* ip = nullptr;
     if (lane < Tc) {
-      prow = P.perm ? P.perm[tok0 + lane] : tok0 + lane;
+      prow = MULTI ? P.perm[tok0 + lane] : tok0 + lane;
       ip = (const char*)(P.idx + prow);
     }
     {
@@ -642,26 +644,32 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   const bool tiled = has_base && B.p[0].base_tiled != 0;
   // (with the base weight in tiles the early half measured slower, not faster)
   const bool early = nprob == 1 && has_base && !tiled && grid <= 2 * dz_cu_count();
-  static std::atomic<unsigned long long> attr_done[21];
+  static std::atomic<unsigned long long> attr_done[72];   // one per kernel: 3 x 12 variants, single and batched
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
-    if (!dz_lds_limit_once(attr_done[slot], f, (int)lds)) return DZ_ELAUNCH;
+    if (!dz_lds_limit_once(attr_done[2 * slot + (nprob > 1)], f, (int)lds)) return DZ_ELAUNCH;
     if (nprob == 1) hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WK32), lds, st, B.p[0]);
     else hipLaunchKernelGGL(bkern, dim3(grid), dim3(64 * WK32), lds, st, B);
     return DZ_OK;
   };
+  // several chunks of tokens (33 .. 128 tokens, always two token tiles): variants of their own
+  const bool multi = B.p[0].nchunk > 1;
   auto pick = [&](auto pre_c) -> int {
     constexpr int PRE_ = decltype(pre_c)::value;
-    const int s0 = 7 * PRE_;
-    if (nprob > 1) {
-      if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0);
-      return tiled ? go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 1)
-                   : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 2);
+    const int s0 = 12 * PRE_;
+    if constexpr (TT == 2) {
+      if (multi) {
+        if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 5, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 5>, s0);
+        if (tiled) return go(dz_mdl32_kernel<BITS, TT, PRE_, 4, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 4>, s0 + 1);
+        return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 3, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 3>, s0 + 2)
+                     : go(dz_mdl32_kernel<BITS, TT, PRE_, 3, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 3>, s0 + 3);
+      }
     }
-    if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0 + 3);
-    if (tiled) return go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 4);
-    return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 1, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 5)
-                 : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 6);
+    if (multi) return DZ_ESHAPE;   // more than 32 tokens always run with two token tiles
+    if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0 + 4);
+    if (tiled) return go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 5);
+    return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 1, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 6)
+                 : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 7);
   };
   int rc = pre == 2 ? pick(std::integral_constant<int, 2>{}) : pre == 1 ? pick(std::integral_constant<int, 1>{})
                                                                        : pick(std::integral_constant<int, 0>{});
@@ -682,6 +690,10 @@ int dz_launch_mdl32_batch(const MdlParams* P0, int nprob, int bits, int pre, hip
   }
   const int nchunk = B.p[0].nchunk, T = P0[0].T;
   if (nchunk < 1 || nchunk > 4) return DZ_ESHAPE;
+  // several chunks of tokens are read through the token order, a single chunk never is: the
+  // kernel variants are compiled for exactly these two cases
+  for (int j = 0; j < nprob; ++j)
+    if ((B.p[j].perm != nullptr) != (nchunk > 1)) return DZ_EINVAL;
   if (bits == 2) return T <= 16 ? launch32<2, 1>(B, nprob, pre, st, ksplit_override) : launch32<2, 2>(B, nprob, pre, st, ksplit_override);
   return T <= 16 ? launch32<4, 1>(B, nprob, pre, st, ksplit_override) : launch32<4, 2>(B, nprob, pre, st, ksplit_override);
 }
