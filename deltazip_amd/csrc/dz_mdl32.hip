@@ -640,11 +640,10 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2 + WK32 * 512;   // activation slices + the token ids
   // single launches of at most one turn (two workgroups per CU) take the variant that requests half
-  // the base tile before the ids are in
+  // the base tile before the ids are in (not over tiles with several chunks of tokens: no gain there)
   const bool tiled = has_base && B.p[0].base_tiled != 0;
-  // (with the base weight in tiles the early half measured slower, not faster)
-  const bool early = nprob == 1 && has_base && !tiled && grid <= 2 * dz_cu_count();
-  static std::atomic<unsigned long long> attr_done[72];   // one per kernel: 3 x 12 variants, single and batched
+  const bool early = nprob == 1 && has_base && grid <= 2 * dz_cu_count();
+  static std::atomic<unsigned long long> attr_done[78];   // one per kernel: 3 x 13 variants, single and batched
   auto go = [&](auto kern, auto bkern, int slot) -> int {
     const void* f = nprob == 1 ? (const void*)kern : (const void*)bkern;
     if (!dz_lds_limit_once(attr_done[2 * slot + (nprob > 1)], f, (int)lds)) return DZ_ELAUNCH;
@@ -656,7 +655,7 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
   const bool multi = B.p[0].nchunk > 1;
   auto pick = [&](auto pre_c) -> int {
     constexpr int PRE_ = decltype(pre_c)::value;
-    const int s0 = 12 * PRE_;
+    const int s0 = 13 * PRE_;
     if constexpr (TT == 2) {
       if (multi) {
         if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 5, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 5>, s0);
@@ -667,7 +666,9 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
     }
     if (multi) return DZ_ESHAPE;   // more than 32 tokens always run with two token tiles
     if (!has_base) return go(dz_mdl32_kernel<BITS, TT, PRE_, 0, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 0>, s0 + 4);
-    if (tiled) return go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 5);
+    if (tiled)
+      return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 2, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 8)
+                   : go(dz_mdl32_kernel<BITS, TT, PRE_, 2, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 2>, s0 + 5);
     return early ? go(dz_mdl32_kernel<BITS, TT, PRE_, 1, true>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 6)
                  : go(dz_mdl32_kernel<BITS, TT, PRE_, 1, false>, dz_mdl32_batch_kernel<BITS, TT, PRE_, 1>, s0 + 7);
   };
