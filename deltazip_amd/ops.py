@@ -453,11 +453,12 @@ def takes_fused_chunks(T: int, S: int) -> bool:
     """Whether a batch above the fused kernel's 128 tokens goes through it in chunks of 128 rather than
     through the matrix-core kernel.  That kernel works on row blocks of up to 256 tokens of one delta
     and needs some 256 x (N / 256) of them to fill the GPU: a few hundred tokens, the more so when
-    they are spread over many deltas, leave most of it idle (5120 x 5120, 2-bit, 256 tokens: 0.13 to
-    0.19 ms in two chunks against 0.18 ms with one delta and 0.57 ms with 64; at 1024 tokens the
-    matrix cores win unless every 16 tokens belong to another delta).  The number of distinct deltas
-    is known on the device only, so the number of slots stands in for it."""
-    return T <= 2 * MAX_TOKENS_FUSED or (T <= 4 * MAX_TOKENS_FUSED and S >= 32)
+    they are spread over many deltas, leave most of it idle (5120 x 5120, 2-bit, tiled base weight;
+    chunks against the matrix-core kernel with 1 / 16 / 64 deltas in the batch: 384 tokens 0.15 / 0.16
+    / 0.21 ms against 0.19 / 0.24 / 0.57 ms; 512 tokens 0.20 / 0.21 / 0.26 against 0.19 / 0.24 / 0.57;
+    768 tokens 0.29 / 0.30 / 0.34 against 0.20 / 0.24 / 0.58).  The number of distinct deltas is
+    known on the device only, so the number of slots stands in for it."""
+    return T <= 3 * MAX_TOKENS_FUSED or (T <= 4 * MAX_TOKENS_FUSED and S >= 16)
 
 
 def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qweight_stacked,
