@@ -62,6 +62,17 @@ def test_layer_protocol(dev):
     oracle_ids = np.array([{0: -1, 11: 0, 12: 1, 13: 2}[i] for i in token_ids])
     ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], oracle_ids)
     assert o.rel_err(out.cpu().numpy(), ref) <= TOL
+    # the layer reads a tiled copy of its base weight (the default); without it: the same bits
+    assert layer.base_tiled is not None and torch.equal(layer.base_tiled, ops.tile_base(base.weight))
+    plain = from_layer(torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.float16), 4,
+                       DeltaConfig(max_deltas=4, max_bitwidth=bits, tile_base_weights=False), ["gate_proj", "up_proj"])
+    assert plain.base_tiled is None
+    with torch.no_grad():
+        plain.base_layer.weight.copy_(p["wb"])
+    for slot in (1, 2, 3):
+        plain.set_delta(slot, bits, layer.qweight_stacked[slot], None, layer.scales_stacked[slot], None, layer.meta_stacked[slot])
+    plain.set_mapping(index_buf, None, None, None, [t])
+    assert torch.equal(plain(p["x"])[0], out)
     # reset a slot: its tokens fall back to the base layer
     layer.reset_delta(2)
     out2, _ = layer(p["x"])
