@@ -85,7 +85,19 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.qweight_stacked = torch.zeros((max_deltas,) + qs, dtype=torch.int32, device=w.device)
         self.meta_stacked = torch.zeros((max_deltas,) + ms, dtype=torch.int16, device=w.device)
         self.scales_stacked = torch.zeros((max_deltas,) + ss, dtype=torch.float16, device=w.device)
-        self.base_tiled = ops.tile_base(w.contiguous()) if delta_config.tile_base_weights and w.is_cuda else None
+        self._tile_base = bool(delta_config.tile_base_weights) and w.is_cuda
+        self.base_tiled = None
+        self.refresh_base_tiles()
+
+    def refresh_base_tiles(self) -> None:
+        """(Re)makes the tiled copy of the base weight that calls of up to 128 tokens read.  Runs when
+        the delta weights are created and again, by itself, when the base weight has been written
+        in place since (its version counter moved); call it after replacing `base_layer.weight`."""
+        if not self._tile_base:
+            return
+        w = self.base_layer.weight
+        self.base_tiled = ops.tile_base(w.detach().contiguous())
+        self._tiled_of = (w.data_ptr(), w._version)
 
     def reset_delta(self, index: int):
         # all-zero scales make the slot contribute exactly 0 whatever the packed words hold
@@ -124,6 +136,9 @@ class LinearWithDelta(BaseLayerWithDelta):
     def apply_weights(self, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         T = self.indices_len[0]
         order = self.token_order[:T] if self.token_order is not None and 32 < T <= ops.MAX_TOKENS_FUSED else None
+        w = self.base_layer.weight
+        if self.base_tiled is not None and self._tiled_of != (w.data_ptr(), w._version):
+            self.refresh_base_tiles()
         return ops.apply_delta(x, self.qweight_stacked, self.scales_stacked, self.meta_stacked,
                                self.indices[:T], self.base_layer.weight, order=order, base_tiled=self.base_tiled)
 

@@ -73,6 +73,14 @@ def test_layer_protocol(dev):
         plain.set_delta(slot, bits, layer.qweight_stacked[slot], None, layer.scales_stacked[slot], None, layer.meta_stacked[slot])
     plain.set_mapping(index_buf, None, None, None, [t])
     assert torch.equal(plain(p["x"])[0], out)
+    # the base weight written in place after the layer was made: the tiles follow
+    with torch.no_grad():
+        base.weight.mul_(2.0)
+    out_w2, _ = layer(p["x"])
+    with torch.no_grad():
+        base.weight.copy_(p["wb"])
+    assert o.rel_err(out_w2.cpu().numpy(), o.forward_ref(p["x_np"], 2 * p["wb_np"], p["dts"], oracle_ids)) <= TOL
+    assert torch.equal(layer(p["x"])[0], out)
     # reset a slot: its tokens fall back to the base layer
     layer.reset_delta(2)
     out2, _ = layer(p["x"])
