@@ -529,13 +529,13 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   if (has_item) {
     f4_t tot = {0.f, 0.f, 0.f, 0.f};
     const int nother = P.nsplit - 1;
-    for (int k0 = 0; k0 < nother; k0 += 8) {
-      unsigned v[8][4];
+    for (int k0 = 0; k0 < nother; k0 += 4) {
+      unsigned v[4][4];
       int spins = 0;
       for (;;) {
         unsigned all = 0xffffffffu;
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
+        for (int u = 0; u < 4; ++u) {
           const unsigned* pp = (const unsigned*)part_ptr(min(k0 + u, nother - 1), wave);
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -548,10 +548,10 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
           if (lane == 0) atomicOr(P.status, 2u);
           break;
         }
-        __builtin_amdgcn_s_sleep(4);
+        __builtin_amdgcn_s_sleep(1);
       }
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < 4; ++u)
         if (k0 + u < nother) {
 #pragma unroll
           for (int e = 0; e < 4; ++e) tot[e] += __builtin_bit_cast(float, v[u][e]);
