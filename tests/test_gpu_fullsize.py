@@ -45,6 +45,9 @@ CASES = [
     # further shapes outside the configurations: 13B layers at decode sizes
     pytest.param(5120, 5120, 2, -1, 64, 128, "uniform", id="13b-5120x5120-T128-D64"),
     pytest.param(13824, 5120, 4, -1, 4, 16, "uniform", id="13b-down-4bit-T16"),
+    # Llama-2-70B MLP layers (one tensor-parallel rank would hold a slice; the whole layer is the larger case)
+    pytest.param(8192, 28672, 4, 128, 2, 100, "uniform", id="70b-8192x28672-4bit-g128-T100"),
+    pytest.param(28672, 8192, 2, -1, 3, 32, "uniform", id="70b-28672x8192-2bit-T32"),
 ]
 
 
