@@ -1,6 +1,7 @@
-// Fused multi-delta linear kernel for decode-sized batches (T <= 32 tokens).
+// Fused multi-delta linear kernel for decode-sized batches: up to 128 tokens per launch, in chunks
+// of 32 (several chunks: the tokens are taken in an order that spreads the deltas over the chunks).
 //
-// One workgroup = 4 wavefronts = one n-pair (32 output rows) x a chunk of k-blocks; each
+// One workgroup = 4 wavefronts = one n-pair (32 output rows) x a slice of k-blocks x one chunk; each
 // wavefront owns whole k-blocks (256 input columns) of that n-pair and is self-sufficient until
 // the final reduction:
 //   * the token ids are fetched first; the distinct deltas of the batch are enumerated
@@ -8,10 +9,11 @@
 //     per-column mask.  Batches that arrive sorted by id (as the reference's scheduler delivers
 //     them) touch fewer column tiles;
 //   * the activations slice goes first (straight into LDS; it does not depend on the ids), then
-//     the packed words of up to 8 deltas (two batches of 4); the base tile is requested once the
-//     first batch has been multiplied, so that a wavefront is not held at its request queue while
-//     data it could work on has arrived.  The number of requests is fixed, so the wait in front
-//     of each use is exact;
+//     the packed words of up to 8 deltas (two batches of 4); the base tile -- row-major or in
+//     16 KiB tiles, streamed or, with several chunks, left in L2 for the next chunk's workgroup --
+//     is requested once the first batch has been multiplied, so that a wavefront is not held at
+//     its request queue while data it could work on has arrived.  The number of requests is
+//     fixed, so the wait in front of each use is exact;
 //   * one read of the dense operand (activations, from the wavefront's own LDS slice) feeds every
 //     delta of the current batch (2:4-sparse v_smfmac_f32_16x16x64_f16, unpacked codes as the
 //     sparse operand, stored positions as its index operand); the base tile follows on
