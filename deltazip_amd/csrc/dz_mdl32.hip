@@ -599,17 +599,16 @@ __global__ __launch_bounds__(64 * WK32, 2) void dz_mdl32_batch_kernel(const MdlB
   mdl32_body<BITS, TT, PRE, BASE, false, false>(B.p[j], npg - first, kc, ch, smem);
 }
 
-// K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each; a
-// launch over the tiled base weight that has one and a half per CU without a split stays unsplit
-// (q + k + v of 4096 rows each: 384 workgroups of four rounds and no partial sums to exchange beat
-// 768 of two rounds: 45.3 against 47.2 us; over the row-major weight the split wins)
+// K split over workgroups: aim at two resident workgroups per CU (512) with few rounds each.  The
+// split depends on the shapes only, not on the form of the base weight: both forms give the same
+// bits.  (q + k + v of 4096 rows each as 384 unsplit workgroups of four rounds instead of 768 of two:
+// the same time over tiles, slower over rows.)
 static int choose_split(const MdlParams& P, int np_total, int ksplit_override) {
   int nsplit = ksplit_override;
   if (nsplit <= 0) {
     nsplit = 1;
     const int max_split = (P.NKB + WK32 - 1) / WK32;  // at least one round of 4 k-blocks each
-    if (!P.base_tiled || (long long)np_total * P.nchunk < 384)
-      while (nsplit < max_split && (long long)np_total * nsplit * P.nchunk < 512) ++nsplit;
+    while (nsplit < max_split && (long long)np_total * nsplit * P.nchunk < 512) ++nsplit;
   }
   if (nsplit > 16 / P.nchunk) nsplit = 16 / P.nchunk;   // the workspace holds 16 sets of partial sums
   if (nsplit > P.NKB) nsplit = P.NKB;

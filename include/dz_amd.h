@@ -250,11 +250,8 @@ int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint
 int dz_tile_base(const uint16_t* w, int K, int N, uint16_t* out, void* stream);
 
 /* dz_multi_delta_linear_batch with every w_base_tiled[j] in the tiled form dz_tile_base writes
- * (ncalls = 1: the single layer call).  The same products in the same order as with the row-major
- * form: bit for bit the same results whenever the two launches split K alike, which they do
- * unless the launch has 384 or more workgroups before any split (N[0] + ... over 32, times the
- * chunks of 32 tokens): over tiles such a launch stays unsplit, and the fp32 sums over K then
- * round as they do between a batched and a separate call. */
+ * (ncalls = 1: the single layer call).  The same products summed in the same order as with the
+ * row-major form: the results are the same, bit for bit. */
 int dz_multi_delta_linear_batch_tiled(int ncalls, const uint16_t* const* x,
                                       const uint16_t* const* w_base_tiled,
                                       const void* const* codes_stacked, const void* const* meta_stacked,

@@ -330,25 +330,16 @@ def test_tiled_base_weight_gives_the_same_bits(dev, n, k, bits, gs, nd, t):
     assert _lib.lib().dz_tile_base(p["wb"].data_ptr(), k - 64, n, tiled.data_ptr(), None) != 0    # whole k-blocks only
 
 
-def test_tiled_base_weight_wide_launch_stays_unsplit(dev):
-    """12288 output rows (q, k and v of a 4096-wide model fused): 384 workgroups before any split.
-    Over tiles the launch stays unsplit in K, over rows it runs two K-slices: the fp32 sums round
-    differently, so the two agree like a batched and a separate call do, and both match the oracle."""
+def test_tiled_base_weight_wide_launch(dev):
+    """12288 output rows (q, k and v of a 4096-wide model fused), split in K: the K split depends on
+    the shapes only, so both forms of the base weight give the same bits here, too."""
     p = make_problem(12288, 2048, 2, -1, 4, 24, "uniform", 77, dev)
     ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
     y0 = run_layer(p)
     y1 = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=ops.tile_base(p["wb"]))
     torch.cuda.synchronize()
-    assert o.rel_err(y0.cpu().numpy(), ref) <= TOL and o.rel_err(y1.cpu().numpy(), ref) <= TOL
-    assert o.rel_err(y1.cpu().numpy(), y0.float().cpu().numpy()) <= 2e-3
-    try:
-        ops.set_ksplit(2)    # the same split on both sides: the same bits again
-        y2 = ops.apply_delta(p["x"], p["q"], p["s"], p["m"], p["ids"], p["wb"], base_tiled=ops.tile_base(p["wb"]))
-        y3 = run_layer(p)
-        torch.cuda.synchronize()
-    finally:
-        ops.set_ksplit(0)
-    assert torch.equal(y2, y3) and torch.equal(y3, y0)
+    assert o.rel_err(y0.cpu().numpy(), ref) <= TOL
+    assert torch.equal(y0, y1)
 
 
 def test_fused_layer_calls_replay_from_a_graph(dev):
