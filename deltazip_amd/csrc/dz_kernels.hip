@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "../../include/dz_amd.h"
+#include "../../include/dz_amd_tuning.h"
 #include <atomic>
 
 #include "dz_device.h"
@@ -499,7 +500,9 @@ __global__ __launch_bounds__(256) void dz_tile_base_kernel(const u4_t* __restric
 // ---------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------
-std::atomic<int> g_ksplit_override{0};
+// K-slice override of the tuning hook (include/dz_amd_tuning.h): per host thread, so that a test
+// or a sweep that sets it changes no other caller's launches
+thread_local int g_ksplit_override = 0;
 
 inline int check_group(int K, int group_size, int* gs_out) {
   int gs = (group_size == -1 || group_size == K) ? K : group_size;
@@ -562,7 +565,7 @@ const char* dz_strerror(int code) {
   }
 }
 
-void dz_set_ksplit(int nsplit) { g_ksplit_override.store(nsplit, std::memory_order_relaxed); }
+void dz_set_ksplit(int nsplit) { g_ksplit_override = nsplit; }
 
 int dz_dequant(const void* codes, const void* meta, const void* scales, int K, int N, int bits,
                int group_size, uint16_t* out, void* stream) {
@@ -791,7 +794,7 @@ static int multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const 
   // groups to the chunks of 32; one launch carries all chunks
   if (T > 32 && !order)
     hipLaunchKernelGGL(dz_deal_kernel, dim3(1), dim3(128), 0, st, (const long long*)indices, T, S, perm);
-  return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override.load(std::memory_order_relaxed));
+  return dz_launch_mdl32_batch(P, ncalls, bits, pre, st, g_ksplit_override);
 }
 
 int dz_multi_delta_linear_batch(int ncalls, const uint16_t* const* x, const uint16_t* const* w_base,

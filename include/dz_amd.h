@@ -321,11 +321,6 @@ int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* c
                         int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
                         uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
 
-/* Debugging and tuning hook, not part of the layer's interface: overrides, for every later call of
- * the process, the number of K-slices of the fused kernel (0 = automatic, the default).  The
- * results do not depend on it beyond the order of the fp32 additions. */
-void dz_set_ksplit(int nsplit);
-
 #ifdef __cplusplus
 }
 #endif

@@ -12,7 +12,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
 def _declared_functions():
-    text = open(os.path.join(ROOT, "include", "dz_amd.h")).read()
+    # the layer's interface and, kept apart from it, the tuning hooks
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in ("dz_amd.h", "dz_amd_tuning.h"))
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(dz_[a-z0-9_]+)\s*\(", text)))
 

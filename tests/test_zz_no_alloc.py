@@ -1,7 +1,9 @@
 """dz_multi_delta_linear_static, the entry point that allocates nothing: its workspace is a fixed
 array inside the library.  Called through the C ABI twice in a row, the second call with a smaller
 input, and compared with dz_multi_delta_linear (bit for bit: same kernels, same order of additions)
-and with the CPU oracle (to the layer's tolerance)."""
+and with the CPU oracle (to the layer's tolerance).  That it allocates nothing is checked as well:
+with the output tensor made beforehand, the device's free memory (hipMemGetInfo) and the bytes
+torch's allocator holds are the same before and after the static calls."""
 import ctypes as C
 
 import numpy as np
@@ -13,10 +15,10 @@ from deltazip_amd import _lib, ops
 from _util import make_problem, TOL
 
 
-def _call(fn_name, p, ws=None, accumulate=0):
+def _call(fn_name, p, ws=None, accumulate=0, out=None):
     L = _lib.lib()
     t, k, n = p["x"].shape[0], p["k"], p["n"]
-    y = torch.full((t, n), 7.0, dtype=torch.float16, device=p["x"].device)
+    y = torch.full((t, n), 7.0, dtype=torch.float16, device=p["x"].device) if out is None else out
     if accumulate:
         y.copy_(p["y0"])
     gs = -1 if p["s"][0].numel() == n else k // (p["s"][0].numel() // n)
@@ -45,14 +47,22 @@ PAIRS = [
 @pytest.mark.gpu
 @pytest.mark.parametrize("big,small", PAIRS)
 def test_static_entry_point_matches_workspace_entry_point(dev, big, small):
-    mem_before = None
     for i, (n, k, bits, gs, nd, t) in enumerate((big, small)):
         p = make_problem(n, k, bits, gs, nd, t, "uniform", 300 + i, dev)
         want = _call("dz_multi_delta_linear", p, ws=_workspace(p))
-        if mem_before is None:
-            mem_before = torch.cuda.memory_allocated()
-        got = _call("dz_multi_delta_linear_static", p)
+        got = _call("dz_multi_delta_linear_static", p)     # first call on the device: looks up the array's address
         assert torch.equal(got, want)
+        # nothing is allocated: neither from the device (hipMalloc would lower the free bytes) nor
+        # from torch's allocator; the output tensor exists before the measurement starts
+        out = torch.empty_like(got)
+        torch.cuda.synchronize()
+        free_before, reserved_before = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+        allocated_before = torch.cuda.memory_allocated()
+        got2 = _call("dz_multi_delta_linear_static", p, out=out.fill_(7.0))
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_reserved() == reserved_before
+        assert torch.cuda.memory_allocated() == allocated_before
+        assert torch.equal(got2, want)
         ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
         assert o.rel_err(got.cpu().numpy(), ref) <= TOL
         # y += result
