@@ -228,7 +228,7 @@ def run_full_step(args, parity):
     multi-delta layer; reports the step, the share of the projections in it and their HBM fraction."""
     from deltazip_amd import DeltaConfig, DeltaMapping, create_delta_manager
     from deltazip_amd.llama_step import LlamaForDecodeStep, LlamaStepConfig
-    from deltazip_amd.synthetic import random_native_stack
+    from deltazip_amd.synthetic import gaussian_native_stack, random_native_stack
     cfg = CONFIGS[5]
     T, S, bits, gs, ctx = cfg["T"], cfg["S"], cfg["bits"], cfg["gs"], 1024
     steps, warmup = args.steps or 10, args.warmup or 2
@@ -239,11 +239,12 @@ def run_full_step(args, parity):
     mgr = create_delta_manager(model, max_num_seqs=T, max_num_batched_tokens=T, vocab_size=mcfg.vocab_size,
                                delta_config=DeltaConfig(max_deltas=S, max_bitwidth=bits, group_size=gs,
                                                         tile_base_weights=not args.row_major_base))
-    # synthetic deltas written straight into the layers' slot stacks (compressing 64 x 32 real deltas
-    # would take hours); the manager is told that delta d + 1 lives in slot d
+    # synthetic deltas (N(0, 1e-3), compressed on the GPU) written straight into the layers' slot stacks;
+    # the manager is told that delta d + 1 lives in slot d
+    make_stack = random_native_stack if args.random_bits else gaussian_native_stack
     for name, layer in mgr.modules.items():
         N, K = layer.base_layer.weight.shape
-        layer.qweight_stacked, layer.meta_stacked, layer.scales_stacked = random_native_stack(K, N, bits, gs, S, dev, gen)
+        layer.qweight_stacked, layer.meta_stacked, layer.scales_stacked = make_stack(K, N, bits, gs, S, dev, gen)
         layer.bitwidth = [bits] * S
     mgr.delta_index_to_id = list(range(1, S + 1))
     ids = torch.sort(torch.randint(1, S + 1, (T,), device=dev, generator=gen)).values.tolist()
@@ -273,7 +274,9 @@ def run_full_step(args, parity):
         "metric": "multi-delta linear tokens/s + achieved HBM TB/s (% peak), Llama-7B shapes",
         "value": T / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": ms_per_step, "ms_per_step_median": round(step_ms[steps // 2], 4), "warmup_steps_run": warm_run,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic (random-init model; " + ("delta slots filled with uniformly random bits)" if args.random_bits
+                                                     else "deltas ~ N(0, 1e-3) compressed on the GPU)"),
         "config": {"workload": cfg["name"] + ", batch sorted by delta id", "baseline_config": 5, "tokens": T,
                    "deltas": S, "deltas_present": d_present, "bits": bits, "group_size": gs, "kv_context": ctx,
                    "layers": mcfg.num_hidden_layers, "launches_per_step": len(projs),
@@ -304,6 +307,10 @@ def main():
                     help="up to 128 tokens: read the base weight as the plain [N, K] tensor instead of the tiled copy "
                          "a layer makes of it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--random-bits", action="store_true",
+                    help="fill the delta slots with uniformly random code and position bits instead of compressing "
+                         "N(0, sigma) deltas (the configured workload)")
+    ap.add_argument("--no-probe", action="store_true", help="skip the read-only yardstick launches")
     ap.add_argument("--ksplit", type=int, default=0)
     ap.add_argument("--separate-launches", action="store_true",
                     help="one launch per projection (default: q/k/v and gate/up, which share their input in a "
@@ -319,7 +326,7 @@ def main():
         print("bench.py needs a GPU (there is no CPU fallback for the measured path)", file=sys.stderr)
         sys.exit(2)
     from deltazip_amd import _lib, ops
-    from deltazip_amd.synthetic import random_native_stack
+    from deltazip_amd.synthetic import gaussian_native_stack, random_native_stack
     cfg = CONFIGS[args.config]
     shapes, T, S, bits, gs = cfg["shapes"], cfg["T"], cfg["S"], cfg["bits"], cfg["gs"]
     steps = args.steps or (10 if args.config == 4 else 200)
@@ -337,24 +344,38 @@ def main():
     # ---- resident inputs
     # up to 128 tokens the layer reads its base weight from the tiled copy it makes at creation
     # (dz_tile_base); --row-major-base measures the fused kernel on the plain [N, K] weight instead
-    tiled_base = T <= 128 and not args.row_major_base
+    fused = T <= 128
+    tiled_base = fused and not args.row_major_base
+    default_workload = (args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
+                        and not args.row_major_base)
     ids = make_ids(cfg["ids"], T, S, dev, gen, not args.unsorted)
     d_present = int(torch.unique(ids).numel())
+    sigma = 2e-3 if args.config == 1 else 1e-3
     layers = []
-    for _ in range(nlayers):
+    for li in range(nlayers):
         calls = []
-        for name, K, N in shapes:
-            q, m, s = random_native_stack(K, N, bits, gs, S, dev, gen)
+        for si, (name, K, N) in enumerate(shapes):
+            if args.random_bits:
+                q, m, s = random_native_stack(K, N, bits, gs, S, dev, gen)
+            else:
+                # the deltas the configuration describes: N(0, sigma), scales from the un-pruned values,
+                # 2:4 by magnitude, quantised -- compressed on the GPU (seeded per configuration, layer, shape)
+                dgen = torch.Generator(device=dev).manual_seed(1000 * args.config + 100 * li + si)
+                q, m, s = gaussian_native_stack(K, N, bits, gs, S, dev, dgen, sigma)
             wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
-            if tiled_base:
-                wb = ops.tile_base(wb)      # as a layer does once when it is created; only this form is read
+            wbt = ops.tile_base(wb) if fused else None     # as a layer does once when it is created
+            if fused and not default_workload:
+                # only one form is read in this run (the default workload also times the other one)
+                if tiled_base:
+                    wb = None
+                else:
+                    wbt = None
             x = torch.randn((T, K), device=dev, generator=gen).half()
             y = torch.empty((T, N), dtype=torch.float16, device=dev)
-            calls.append((name, K, N, x, wb, q, m, s, y))
+            calls.append((name, K, N, x, wb, q, m, s, y, wbt))
         layers.append(calls)
     stream = torch.cuda.current_stream().cuda_stream
     ops.set_ksplit(args.ksplit)
-    fused = T <= 128
 
     # launches of a step: q/k/v in one, o, gate/up in one, down (the reference runs q/k/v and gate/up as
     # fused layers: serving/vllm/delta/layers_marlin.py:281-487); --separate-launches: one per projection
@@ -363,79 +384,68 @@ def main():
     if fused and not args.separate_launches and names == [sh[0] for sh in SHAPES]:
         groups = [[0, 1, 2], [3], [4, 5], [6]]
 
+    vp = C.c_void_p
+    keep = []                                   # the pointer arrays must outlive the calls
     if fused:
-        # pre-marshalled C-ABI calls (device pointers and sizes only)
         ws_bytes = max(lib.dz_workspace_bytes(T, shapes[g[0]][1], sum(shapes[j][2] for j in g)) for g in groups)
         ws = torch.zeros(ws_bytes, dtype=torch.uint8, device=dev)
-        f = lib.dz_multi_delta_linear
-        fb = lib.dz_multi_delta_linear_batch_tiled if tiled_base else lib.dz_multi_delta_linear_batch
-        vp = C.c_void_p
         # 33..128 tokens: the order in which the kernel takes the tokens depends on the ids only; it is
         # computed once per step (inside the timed region) and every launch of the step reuses it, as the
         # reference converts its mapping once per batch
         order = torch.empty(T, dtype=torch.int32, device=dev) if T > 32 else None
-        keep = []                                   # the pointer arrays must outlive the calls
-        prepared = []
-        single = []                                 # every projection as a launch of its own (per-shape timing)
-        for calls in layers:
-            pc = []
-            for g in groups:
-                if len(g) == 1 and order is None and not tiled_base:
-                    name, K, N, x, wb, q, m, s, y = calls[g[0]]
-                    pc.append((f, (vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()),
-                                   vp(s.data_ptr()), vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
-                                   vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))))
-                else:
+
+        def marshal(tiled, ids_t):
+            """Pre-marshalled C-ABI calls (device pointers and sizes only): per layer the launches of a
+            step, and every projection as a launch of its own (per-shape timing)."""
+            fb = lib.dz_multi_delta_linear_batch_tiled if tiled else lib.dz_multi_delta_linear_batch
+            prepared, single = [], []
+            for calls in layers:
+                def batch_args(g):
                     n = len(g)
                     arr = lambda k: (vp * n)(*[calls[j][k].data_ptr() for j in g])
-                    ax, aw, aq, am, asc, ay = arr(3), arr(4), arr(5), arr(6), arr(7), arr(8)
+                    ax, aw, aq, am, asc, ay = arr(3), arr(9 if tiled else 4), arr(5), arr(6), arr(7), arr(8)
                     an = (C.c_int * n)(*[calls[j][2] for j in g])
                     keep.append((ax, aw, aq, am, asc, ay, an))
-                    pc.append((fb, (n, ax, aw, aq, am, asc, vp(ids.data_ptr()), ay, an, an, T, calls[g[0]][1], S, bits,
-                                    gs, 0, vp(order.data_ptr()) if order is not None else None,
-                                    vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))))
-            prepared.append(pc)
-            if tiled_base:
-                one = []
-                for name, K, N, x, wb, q, m, s, y in calls:
-                    a1 = [(vp * 1)(t.data_ptr()) for t in (x, wb, q, m, s, y)]
-                    an = (C.c_int * 1)(N)
-                    keep.append((a1, an))
-                    one.append((1, a1[0], a1[1], a1[2], a1[3], a1[4], vp(ids.data_ptr()), a1[5], an, an, T, K, S, bits, gs, 0,
-                                None, vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream)))
-                single.append(one)
-            else:
-                single.append([(vp(x.data_ptr()), vp(wb.data_ptr()), vp(q.data_ptr()), vp(m.data_ptr()), vp(s.data_ptr()),
-                                vp(ids.data_ptr()), vp(y.data_ptr()), T, K, N, S, bits, gs, 0, N,
-                                vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))
-                               for name, K, N, x, wb, q, m, s, y in calls])
+                    return (n, ax, aw, aq, am, asc, vp(ids_t.data_ptr()), ay, an, an, T, calls[g[0]][1], S, bits,
+                            gs, 0, vp(order.data_ptr()) if order is not None else None,
+                            vp(ws.data_ptr()), C.c_size_t(ws_bytes), vp(stream))
+                prepared.append([(fb, batch_args(g)) for g in groups])
+                single.append([(fb, batch_args([j])) for j in range(len(calls))])
+            return prepared, single
 
-        def launch(i, gi):
-            fn, a = prepared[i % len(prepared)][gi]
+        prepared, single = marshal(tiled_base, ids)
+
+        def launch(i, gi, prep=None):
+            fn, a = (prep or prepared)[i % len(layers)][gi]
             rc = fn(*a)
             if rc:
                 raise RuntimeError(f"multi-delta linear launch failed: {lib.dz_strerror(rc).decode()}")
 
         def call(i, idx):
-            rc = (fb if tiled_base else f)(*single[i % len(single)][idx])
-            if rc:
-                raise RuntimeError(f"dz_multi_delta_linear failed: {lib.dz_strerror(rc).decode()}")
+            launch(i, idx, single)
     else:
         # prefill-sized: the host wrapper groups the batch and runs the packed-delta GEMM
+        order = None
+
         def call(i, idx):
-            name, K, N, x, wb, q, m, s, y = layers[i % len(layers)][idx]
+            name, K, N, x, wb, q, m, s, y, _ = layers[i % len(layers)][idx]
             ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y)
 
-        def launch(i, gi):
+        def launch(i, gi, prep=None):
             call(i, groups[gi][0])
 
-    def step(i):
-        if fused and order is not None:
-            rc = lib.dz_token_order(C.c_void_p(ids.data_ptr()), T, S, C.c_void_p(order.data_ptr()), C.c_void_p(stream))
-            if rc:
-                raise RuntimeError(f"dz_token_order failed: {lib.dz_strerror(rc).decode()}")
-        for gi in range(len(groups)):
-            launch(i, gi)
+    def make_step(prep=None, ids_t=None):
+        ids_t = ids if ids_t is None else ids_t
+
+        def step(i):
+            if fused and order is not None:
+                rc = lib.dz_token_order(C.c_void_p(ids_t.data_ptr()), T, S, C.c_void_p(order.data_ptr()), C.c_void_p(stream))
+                if rc:
+                    raise RuntimeError(f"dz_token_order failed: {lib.dz_strerror(rc).decode()}")
+            for gi in range(len(groups)):
+                launch(i, gi, prep)
+        return step
+    step = make_step()
 
     if args.calib_copy_mib > 0:
         src = torch.ones(args.calib_copy_mib << 19, dtype=torch.float16, device=dev)
@@ -450,8 +460,6 @@ def main():
 
     def abytes(K, N):
         return algorithmic_bytes(K, N, T, bits, d_present, 1 if gs == -1 else K // gs)
-    default_workload = (args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
-                        and not args.row_major_base)
     launches = steps * len(groups)
     step_bytes = sum(abytes(K, N) for _, K, N in shapes)
     step_flops = sum(2.0 * T * K * N for _, K, N in shapes)
@@ -475,6 +483,19 @@ def main():
                    "frac": round(2.0 * T * K * N / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 3)}
         per_call_us[f"{K}x{N}"] = ent
 
+    def time_loop(fn, iters, warm=12):
+        """us per call of fn(i) over `iters` back-to-back calls on the current stream (HIP events)."""
+        for i in range(warm):
+            fn(i)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(iters):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / iters
+
     if cfg["bound"] == "hbm":
         achieved = (step_bytes / len(groups)) / avg_launch_s / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
@@ -485,6 +506,77 @@ def main():
                     "kernel": "dz_mdl32_kernel" if all(len(g) == 1 for g in groups) else "dz_mdl32_kernel + dz_mdl32_batch_kernel (same body)",
                     "algorithmic_bytes_per_launch": step_bytes // len(groups),
                     "avg_launch_us": round(avg_launch_s * 1e6, 2)}
+        if default_workload:
+            # the two qualifiers of the headline, measured in the same run on the same weights: the batch
+            # as drawn (not sorted by delta id), and the base weight read as the plain [N, K] tensor
+            reps = max(50, min(steps, 200))
+            ids_u = make_ids(cfg["ids"], T, S, dev, torch.Generator(device=dev).manual_seed(1234), False)
+            prep_u, _ = marshal(True, ids_u)
+            us_u = time_loop(make_step(prep_u, ids_u), reps)
+            prep_r, _ = marshal(False, ids)
+            us_r = time_loop(make_step(prep_r), reps)
+            roofline["unsorted_frac"] = round(step_bytes / us_u / 1e3 / HBM_PEAK_GBPS, 4)
+            roofline["row_major_frac"] = round(step_bytes / us_r / 1e3 / HBM_PEAK_GBPS, 4)
+            roofline["unsorted_ms_per_step"] = round(us_u * 1e-3, 5)
+            roofline["row_major_ms_per_step"] = round(us_r * 1e-3, 5)
+        if fused and tiled_base and T <= 32 and not args.no_probe and all(len(g) <= 4 for g in groups):
+            # Yardstick: for every launch of the step, a read-only launch with the same grid that makes
+            # the same 16-byte streaming requests for the tiled base weight and the packed words of the
+            # deltas present -- no ids, no arithmetic, no exchange of partial sums, no output -- and
+            # the fused launch timed the same way (back to back, rotating over the resident layers).
+            sink = torch.zeros(64, dtype=torch.int32, device=dev)
+            dpr = min(d_present, 8)
+            pp = {}
+            pargs = []
+            for gi, g in enumerate(groups):
+                pa = []
+                for calls in layers:
+                    n = len(g)
+                    arr = lambda k: (vp * n)(*[calls[j][k].data_ptr() for j in g])
+                    ax, aw, aq, am = arr(3), arr(9), arr(5), arr(6)
+                    an = (C.c_int * n)(*[calls[j][2] for j in g])
+                    keep.append((ax, aw, aq, am, an))
+                    pa.append((n, ax, aw, aq, am, an, T, shapes[g[0]][1], bits, dpr))
+                pargs.append(pa)
+
+            def probe(i, gi, with_x):
+                rc = lib.dz_probe_read(*pargs[gi][i % len(layers)], with_x, vp(sink.data_ptr()), vp(stream))
+                if rc:
+                    raise RuntimeError(f"dz_probe_read failed: {lib.dz_strerror(rc).decode()}")
+
+            def probe_step(i, with_x):
+                for gi in range(len(groups)):
+                    probe(i, gi, with_x)
+            # the whole step as read-only launches, in the step's own order over the same resident layers
+            # (same footprint per pass as the timed loop: nothing is found in the last-level cache)
+            reps = max(50, min(steps, 200))
+            probe_step_us = {wx: time_loop(lambda i: probe_step(i, wx), reps) for wx in (0, 1)}
+            fused_step_us = time_loop(step, reps)
+            for gi, g in enumerate(groups):
+                K = shapes[g[0]][1]
+                wbytes = sum(2 * K * shapes[j][2] + dpr * (K * shapes[j][2] * bits // 16 + K * shapes[j][2] // 8) for j in g)
+                abytes_g = sum(abytes(shapes[j][1], shapes[j][2]) for j in g)
+                us0 = time_loop(lambda i: probe(i, gi, 0), 60)
+                us1 = time_loop(lambda i: probe(i, gi, 1), 60)
+                usf = time_loop(lambda i: launch(i, gi), 60)
+                pp["+".join(names[j] for j in g)] = {
+                    "weight_bytes": wbytes, "algorithmic_bytes": abytes_g,
+                    "read_only_us": round(us0, 2), "read_only_frac_of_peak": round(wbytes / us0 / 1e3 / HBM_PEAK_GBPS, 4),
+                    "read_only_with_activation_requests_us": round(us1, 2),
+                    "fused_us": round(usf, 2), "fused_frac_of_peak": round(abytes_g / usf / 1e3 / HBM_PEAK_GBPS, 4),
+                    "fused_over_read_only": round(us0 / usf, 4)}
+            roofline["practical_peak"] = {
+                "what": "read-only launches with the fused kernel's grids and 16-byte streaming requests (dz_probe_read): "
+                        "no ids, no arithmetic, no exchange, no output; each launch timed back to back like the fused one",
+                "per_launch_note": "each launch repeated back to back over the resident layers: a smaller footprint per "
+                                   "pass than the step's, so part of it may be found in the last-level cache; the step "
+                                   "figures below are the yardstick",
+                "per_launch": pp,
+                "step_read_only_us": round(probe_step_us[0], 2),
+                "step_read_only_with_activation_requests_us": round(probe_step_us[1], 2),
+                "step_fused_us": round(fused_step_us, 2),
+                "frac": round(step_bytes / probe_step_us[0] / 1e3 / HBM_PEAK_GBPS, 4),
+                "fused_over_read_only": round(probe_step_us[0] / fused_step_us, 4)}
     else:
         # base contraction only (2*T*K*N per call); the per-delta dequantisation and the delta half of
         # the pair-GEMM are extra work inside the same time
@@ -503,7 +595,10 @@ def main():
         "ms_per_step_median": round(median_step_ms, 5), "ms_per_step_min": round(step_ms[0], 5),
         "warmup_steps_run": warm_steps_run,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16",
+        "data": "synthetic" + (" (delta slots filled with uniformly random bits)" if args.random_bits else
+                               " (deltas ~ N(0, %g) compressed on the GPU: scales from the un-pruned values, 2:4 by "
+                               "magnitude, %d-bit codes; base ~ N(0, 0.02), x ~ N(0, 1))" % (sigma, bits)),
         "config": {"workload": cfg["name"] + ("" if args.unsorted or cfg["ids"] in ("zeros", "blocks")
                                               else ", batch sorted by delta id"),
                    "baseline_config": args.config, "tokens": T, "deltas": S, "deltas_present": d_present,

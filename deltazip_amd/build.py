@@ -14,7 +14,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libdz_amd.so")
 
-SOURCES = ["dz_repack.cpp", "dz_kernels.hip", "dz_mdl32.hip", "dz_gemm.hip", "dz_gemm24.hip", "dz_obs.hip"]
+SOURCES = ["dz_repack.cpp", "dz_kernels.hip", "dz_mdl32.hip", "dz_gemm.hip", "dz_gemm24.hip", "dz_obs.hip", "dz_probe.hip"]
 
 # packed fp32 VALU instructions are switched off for every device compilation in this project
 HIPCC_FLAGS = [

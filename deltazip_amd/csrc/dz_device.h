@@ -171,3 +171,4 @@ inline int dz_cu_count() {
 // Launch of the T <= 32 kernel (dz_mdl32.hip).
 int dz_launch_mdl32(const MdlParams& P, int bits, int pre, hipStream_t st, int ksplit_override);
 int dz_launch_mdl32_batch(const MdlParams* P, int nprob, int bits, int pre, hipStream_t st, int ksplit_override);
+void dz_mdl32_geometry(const MdlParams* P, int nprob, int ksplit_override, int* nsplit, int* cb, int* grid);

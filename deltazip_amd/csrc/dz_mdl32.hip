@@ -615,17 +615,30 @@ static int choose_split(const MdlParams& P, int np_total, int ksplit_override) {
   return nsplit;
 }
 
+}  // namespace
+
+// Launch geometry of the fused kernel for a batch of calls (P[j].NP, NKB and nchunk set): K is
+// split as far as the launch needs to fill the GPU -- a batch counts the n-pairs of all its calls
+// (gate + up together fill it without a split, and then exchange no partial sums at all).
+// K-slices need not be whole rounds of WK32 k-blocks: a wavefront without a k-block in a slice's
+// last round idles; the slices are of equal length up to one k-block.
+void dz_mdl32_geometry(const MdlParams* P, int nprob, int ksplit_override, int* nsplit_out, int* cb_out, int* grid_out) {
+  int np_all = 0;
+  for (int j = 0; j < nprob; ++j) np_all += P[j].NP;
+  const int nsplit0 = choose_split(P[0], np_all, ksplit_override);
+  const int cb = (P[0].NKB + nsplit0 - 1) / nsplit0;
+  const int nsplit = (P[0].NKB + cb - 1) / cb;
+  *nsplit_out = nsplit;
+  *cb_out = cb;
+  *grid_out = (np_all + 7) / 8 * 8 * nsplit * P[0].nchunk;
+}
+
+namespace {
+
 template <int BITS, int TT>
 int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override) {
-  // K is split as far as the launch needs to fill the GPU: a batch counts the n-pairs of all its
-  // calls (gate + up together fill it without a split, and then exchange no partial sums at all)
-  int np_all = 0;
-  for (int j = 0; j < nprob; ++j) np_all += B.p[j].NP;
-  const int nsplit0 = choose_split(B.p[0], np_all, ksplit_override);
-  int cb = (B.p[0].NKB + nsplit0 - 1) / nsplit0;
-  // (K-slices need not be whole rounds of WK32 k-blocks: a wavefront without a k-block in a
-  // slice's last round idles; rounding the slice length up leaves the last slice short instead)
-  const int nsplit = (B.p[0].NKB + cb - 1) / cb;
+  int nsplit, cb, grid;
+  dz_mdl32_geometry(B.p, nprob, ksplit_override, &nsplit, &cb, &grid);
   int np_total = 0;
   bool has_base = B.p[0].wb != nullptr;
   for (int j = 0; j < DZ_MAX_BATCH; ++j) {
@@ -638,7 +651,6 @@ int launch32(MdlBatch B, int nprob, int pre, hipStream_t st, int ksplit_override
     }
     B.np_end[j] = np_total;
   }
-  const int grid = (np_total + 7) / 8 * 8 * nsplit * B.p[0].nchunk;
   const size_t lds = (size_t)WK32 * 16 * TT * DZ_KBLOCK * 2 + WK32 * 512;   // activation slices + the token ids
   // single launches of at most one turn (two workgroups per CU) take the variant that requests half
   // the base tile before the ids are in (not over tiles with several chunks of tokens: no gain there)

@@ -1,9 +1,16 @@
-"""Synthetic deltas generated directly in the native layout, on the device.
+"""Synthetic deltas in the native layout, made on the device.
 
-For benchmarks and full-size tests, where compressing real fp32 deltas on the host (a few seconds
-per 4096 x 4096 matrix) would dominate the run.  Every group of four input columns gets a valid,
-uniformly chosen pair of kept positions; codes are uniform random bits; scales are uniform in
-[2e-4, 1.2e-3), the range symmetric 2..4-bit quantisation of sigma = 1e-3 deltas produces.
+`gaussian_native_stack` is the workload the benchmark configurations describe: every delta is
+drawn from N(0, sigma), its scales come from the un-pruned values, it is pruned 2:4 by magnitude
+and quantised (`ops.compress_delta`, byte-identical to the reference's pipeline followed by the
+repacker).  Such deltas have most kept codes at or next to the zero-point and scales tied to the
+row maximum.  The benchmark and the full-size parity tests use it.
+
+`random_native_stack` fills the layout with uniformly random bits instead (every group of four
+input columns gets a valid, uniformly chosen pair of kept positions; codes are uniform; scales
+uniform in [2e-4, 1.2e-3)): every code and position value occurs equally often, which is what
+the layout and arithmetic tests want, and it needs no fp32 delta (64 resident deltas of a whole
+model are filled in seconds).
 """
 from __future__ import annotations
 
@@ -29,3 +36,21 @@ def random_native_stack(K: int, N: int, bits: int, group_size: int, num_deltas: 
     m = torch.where(w >= 2 ** 31, w - 2 ** 32, w).to(torch.int32).view(torch.int16).view((num_deltas,) + ms)
     s = (torch.rand((num_deltas,) + ss, device=device, generator=generator) * 1e-3 + 2e-4).half()
     return q, m, s
+
+
+def gaussian_native_stack(K: int, N: int, bits: int, group_size: int, num_deltas: int, device,
+                          generator: torch.Generator, sigma: float = 1e-3, return_deltas: bool = False):
+    """(qweight_stacked, meta_stacked, scales_stacked) for `num_deltas` slots, each the compressed
+    form of its own delta ~ N(0, sigma) [N, K] fp32 (drawn on the device from `generator`).
+    return_deltas: also the fp32 deltas, as a list (for checks against the CPU restatement)."""
+    qs, ms, ss = ops.stacked_shapes(K, N, bits, group_size)
+    q = torch.empty((num_deltas,) + qs, dtype=torch.int32, device=device)
+    m = torch.empty((num_deltas,) + ms, dtype=torch.int16, device=device)
+    s = torch.empty((num_deltas,) + ss, dtype=torch.float16, device=device)
+    deltas = []
+    for d in range(num_deltas):
+        delta = torch.randn((N, K), device=device, dtype=torch.float32, generator=generator) * sigma
+        q[d], m[d], s[d] = ops.compress_delta(delta, bits, group_size)
+        if return_deltas:
+            deltas.append(delta)
+    return (q, m, s, deltas) if return_deltas else (q, m, s)

@@ -61,7 +61,7 @@ def test_static_entry_point_matches_workspace_entry_point(dev, big, small):
         got2 = _call("dz_multi_delta_linear_static", p, out=out.fill_(7.0))
         assert torch.cuda.mem_get_info()[0] == free_before
         assert torch.cuda.memory_reserved() == reserved_before
-        assert torch.cuda.memory_allocated() == allocated_before
+        assert torch.cuda.memory_allocated() <= allocated_before     # (a temporary of the test itself may have gone)
         assert torch.equal(got2, want)
         ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
         assert o.rel_err(got.cpu().numpy(), ref) <= TOL
