@@ -116,10 +116,15 @@ struct MdlBatch {
 
 constexpr int XS = DZ_KBLOCK + 8;  // LDS row stride of the staged activations, in halves
 
+// Packed words of one delta for one (n-pair, k-block): 16 bytes of positions and NCODE x 16 bytes of
+// codes per lane.  NLOADS is the number of requests load_frag makes; the kernels' hand-written
+// wait counts are built from it, so the two cannot drift apart.
 template <int BITS>
 struct Frag {
+  static constexpr int NCODE = BITS == 2 ? 1 : 2;
+  static constexpr int NLOADS = 1 + NCODE;
   u4_t meta;
-  u4_t code[BITS == 2 ? 1 : 2];
+  u4_t code[NCODE];
 };
 
 template <int BITS>
@@ -131,14 +136,10 @@ __device__ __forceinline__ Frag<BITS> load_frag(const MdlParams& P, int d, int n
   const unsigned lo = (unsigned)lane * 16u;
   const char* mb = (const char*)(P.meta + (size_t)d * P.meta_slot_u4 + tile * 64);
   f.meta = __builtin_nontemporal_load((const u4_t*)(mb + lo));
-  if (BITS == 2) {
-    const char* cb = (const char*)(P.codes + (size_t)d * P.codes_slot_u4 + tile * 64);
-    f.code[0] = __builtin_nontemporal_load((const u4_t*)(cb + lo));
-  } else {
-    const char* cb = (const char*)(P.codes + (size_t)d * P.codes_slot_u4 + tile * 128);
-    f.code[0] = __builtin_nontemporal_load((const u4_t*)(cb + lo));
-    f.code[BITS == 2 ? 0 : 1] = __builtin_nontemporal_load((const u4_t*)(cb + lo + 1024));
-  }
+  // one request per 1 KiB of codes: exactly Frag<BITS>::NCODE of them
+  const char* cb = (const char*)(P.codes + (size_t)d * P.codes_slot_u4 + tile * (64 * Frag<BITS>::NCODE));
+#pragma unroll
+  for (int c = 0; c < Frag<BITS>::NCODE; ++c) f.code[c] = __builtin_nontemporal_load((const u4_t*)(cb + lo + 1024 * c));
   return f;
 }
 

@@ -47,6 +47,13 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   constexpr int TP = 16 * TT;              // padded token count (16 or 32)
   constexpr int G = (BITS == 2) ? (PRE == 2 ? 3 : 4) : (TT == 2 ? 2 : 3);   // deltas per batch (two batches are in flight); 3 where 4 would not fit the registers
   constexpr int NX = TP / 2;               // activation loads per wavefront (2 rows each)
+  // Requests per unit, from which the hand-written wait counts below are built (the request loops
+  // run over the same constants): a delta batch = G x (positions, codes, PRE scale words); one row
+  // fragment of the base tile = 4 steps x 2 halves.
+  constexpr int BATCH_LOADS = G * (Frag<BITS>::NLOADS + PRE);
+  constexpr int BASE_FRAG_LOADS = 4 * 2;
+  constexpr int EARLY_LOADS = EARLY ? BASE_FRAG_LOADS : 0;   // EARLY: fragment 0 goes out with the activations
+  static_assert(NX + 2 * BATCH_LOADS + 2 * BASE_FRAG_LOADS <= 63, "more requests in flight than vmcnt can count");
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wavefront-uniform, in a scalar register
   const int jj = lane & 15, ga = lane >> 4;
@@ -118,6 +125,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
   // bytes.  The matrix instruction wants row jj in lane jj, so before use the upper eight lanes of
   // each group of 16 trade places between the two halves (`base_operands`).
   auto issue_base = [&](int kb, int lane_r, const int s_lo, const int s_hi) {   // row fragments s_lo .. s_hi - 1
+    static_assert(sizeof(a[0]) / sizeof(u4_t) == BASE_FRAG_LOADS, "one request per 16-byte register group of a row fragment");
     if constexpr (TILED) {
       // the tile is 16 requests of 1 KiB, each already in the order the matrix instruction takes
       const char* tb = (const char*)P.wb + dz_base_tile_offset(np, kb, P.NKB) + ((size_t)lane_r << 4);
@@ -215,7 +223,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
       // nothing of the compiler's between the two waits: a scalar load scheduled in there would
       // be waited for by the lgkmcnt(0) below instead of behind the ids' latency
       __builtin_amdgcn_sched_barrier(0);
-      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NX + (EARLY ? 8 : 0)) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" : : "n"(NX + EARLY_LOADS) : "memory");
     }
     {
       unsigned lo, hi;   // read and wait in one statement
@@ -298,8 +306,9 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
           const int ls = real ? lane_r : 0;
           const int gb0 = (kb * DZ_KBLOCK) / P.gs + (ls >> 5);
           const _Float16* sb = P.scales + (size_t)(kd - 1) * P.scales_slot + n0 + (ls & 31);
-          rs[g][0] = *(const unsigned short*)(sb + (size_t)min(gb0, P.G - 1) * P.N);
-          if (PRE == 2) rs[g][1] = *(const unsigned short*)(sb + (size_t)min(gb0 + 2, P.G - 1) * P.N);
+#pragma unroll
+          for (int i = 0; i < PRE; ++i)   // PRE requests: scale groups gb0 (and gb0 + 2 for groups of 64)
+            rs[g][i] = *(const unsigned short*)(sb + (size_t)min(gb0 + 2 * i, P.G - 1) * P.N);
         }
       }
     };
@@ -313,7 +322,7 @@ __device__ __forceinline__ void mdl32_body(const MdlParams& P, const int np, con
     // after them can be outstanding, this wavefront's LDS slice is complete.  (The compiler does
     // not order LDS reads after LDS-direct loads by itself.)
     {
-      constexpr int later = 2 * G * ((BITS == 2 ? 2 : 3) + PRE) + (EARLY ? 8 : 0);   // both batches: words and, with PRE, scales; the early half of the base tile
+      constexpr int later = 2 * BATCH_LOADS + EARLY_LOADS;   // both batches: words and, with PRE, scales; the early fragment of the base tile
       // s_waitcnt immediate on gfx9: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] << 14
       // lgkmcnt(0) as well: the compiler books an LDS-direct load on both counters and, while it
       // believes one outstanding, turns every later vmcnt wait into vmcnt(0)

@@ -88,16 +88,37 @@ class LinearWithDelta(BaseLayerWithDelta):
         self._tile_base = bool(delta_config.tile_base_weights) and w.is_cuda
         self.base_tiled = None
         self.refresh_base_tiles()
+        self._wrap_weight_loader()
 
     def refresh_base_tiles(self) -> None:
-        """(Re)makes the tiled copy of the base weight that calls of up to 128 tokens read.  Runs when
-        the delta weights are created and again, by itself, when the base weight has been written
-        in place since (its version counter moved); call it after replacing `base_layer.weight`."""
+        """(Re)makes the tiled copy of the base weight that calls of up to 128 tokens read.  It runs
+        when the delta weights are created; again, by itself, when the weight tensor has been
+        replaced or written in place through autograd-visible ops (`weight.mul_()`, `weight.copy_()`
+        under no_grad: the tensor's version counter moves); and after every call of the parameter's
+        `weight_loader`, the way the serving engine loads and swaps base weights
+        (model_executor/layers/linear.py:231, 305, 442, 616).  A write that bypasses all three --
+        `weight.data.copy_()` from user code leaves the version counter where it was -- cannot be seen
+        from here: call this method after it (or `DeltaModelManager.refresh_base_weights()`)."""
         if not self._tile_base:
             return
         w = self.base_layer.weight
         self.base_tiled = ops.tile_base(w.detach().contiguous())
         self._tiled_of = (w.data_ptr(), w._version)
+
+    def _wrap_weight_loader(self) -> None:
+        """The engine's loaders write `param.data` (no version bump): a loader that a base parameter
+        carries is wrapped so that the tiled copy follows every load."""
+        w = self.base_layer.weight
+        loader = getattr(w, "weight_loader", None)
+        if loader is None or getattr(loader, "_refreshes_base_tiles", False):
+            return
+
+        def weight_loader(*args, **kwargs):
+            out = loader(*args, **kwargs)
+            self.refresh_base_tiles()
+            return out
+        weight_loader._refreshes_base_tiles = True
+        w.weight_loader = weight_loader
 
     def reset_delta(self, index: int):
         # all-zero scales make the slot contribute exactly 0 whatever the packed words hold

@@ -244,6 +244,9 @@ class DeltaModelManager:
                     raise ValueError(f"{x} is not in list")     # what list.index raises in the reference
         if self._staged is not None:
             self._staged.synchronize()      # the previous transfer has read the staging buffers
+        # the kernels' status words (a delta id out of range; a partial sum that did not arrive): the
+        # copy started at the previous batch is looked at, the next one is started -- no wait of its own
+        ops.poll_status(self.device)
         if self._slots_dirty:
             self._slots_host.copy_(torch.tensor([d if d is not None else 0 for d in self.delta_index_to_id],
                                                 dtype=torch.long))
@@ -263,6 +266,20 @@ class DeltaModelManager:
             ops.token_order(self.base_indices[:T], self.delta_slots, out=self.token_order)
         # the layers keep a reference to this list
         self.indices_len[:] = (T, P, P, T)
+
+    def refresh_base_weights(self) -> None:
+        """Re-tiles the base weight of every delta layer: for callers that have written base weights
+        in a way the layers cannot see (`weight.data.copy_()`), e.g. after swapping the base model."""
+        for module in self.modules.values():
+            if isinstance(module, LinearWithDelta):
+                module.refresh_base_tiles()
+
+    def check_status(self) -> None:
+        """Looks at the kernels' status words now (synchronises with the stream the layers run on):
+        raises `ops.DeltaKernelError` if a launch since the last look reported an invalid output, warns
+        once about delta ids out of range.  `set_delta_mapping` does the same for the previous batch
+        without waiting; this is for a point of the caller's choosing (end of a step, shutdown)."""
+        ops.poll_status(self.device, wait=True)
 
     def set_delta_mapping(self, delta_mapping: DeltaMapping) -> None:
         if self._last_mapping != delta_mapping:

@@ -394,26 +394,117 @@ def map_ids(token_ids: torch.Tensor, prompt_ids: Optional[torch.Tensor], slot_id
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
+WS_HEADER_BYTES = 256          # the status word sits in front of the token order and the partial sums
+
+STATUS_BAD_ID = 1              # a delta id outside [-1, S) was met and treated as -1
+STATUS_SUM_MISSING = 2         # a partial sum of a K-slice did not arrive: that call's output is invalid
+
+
 def _workspace(device: torch.device, T: int, K: int, N: int) -> torch.Tensor:
     need = _lib.lib().dz_workspace_bytes(T, K, N)
     idx = device.index if device.index is not None else torch.cuda.current_device()
     key = (idx, _stream())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
+        new = torch.zeros(max(need, 1 << 20), dtype=torch.uint8, device=device)
+        if ws is not None:
+            # the status word of the buffer that is left behind is carried over (same stream: after
+            # the calls that may still set it)
+            new[:WS_HEADER_BYTES].copy_(ws[:WS_HEADER_BYTES])
+        _workspaces[key] = ws = new
+        _status_polls.pop(key, None)
     return ws
 
 
 def workspace_status(device=None) -> int:
     """Status words of the device's workspaces, OR-ed (bit 0: a delta id outside [-1, S) was seen
-    and treated as -1).  Synchronises; meant for debugging and tests."""
+    and treated as -1; bit 1: a partial sum did not arrive).  Synchronises; meant for debugging
+    and tests -- the serving path uses `poll_status`."""
     idx = torch.cuda.current_device() if device is None else torch.device(device).index
     status = 0
     for (i, _), ws in _workspaces.items():
         if i == idx:
             status |= int(ws[:4].view(torch.int32).item())
     return status
+
+
+class DeltaKernelError(RuntimeError):
+    """A launch of the fused kernel reported that its output is invalid."""
+
+
+_warned_bad_id = False
+
+
+def raise_for_status(word: int, where: str = "multi-delta linear") -> None:
+    """What a status word means to the caller.  Bit 1 -> DeltaKernelError (a RuntimeError, as every
+    failure of the reference's ops is a Python exception); bit 0 -> one warning per process."""
+    global _warned_bad_id
+    if word & STATUS_SUM_MISSING:
+        raise DeltaKernelError(
+            f"{where}: a partial sum of a K dimension split over workgroups did not arrive within the kernel's "
+            "bounded wait; the outputs of the calls since the last check are invalid (status bit 1). The "
+            "workspace has been cleared; repeat the step.")
+    if word & STATUS_BAD_ID and not _warned_bad_id:
+        _warned_bad_id = True
+        import warnings
+        warnings.warn(f"{where}: a delta id outside [-1, S) was met and served as -1 (base weight only; status bit 0)",
+                      RuntimeWarning, stacklevel=3)
+
+
+# (device, stream) -> (pinned int32[1], event of the copy that fills it)
+_status_polls: Dict[Tuple[int, int], Tuple[torch.Tensor, "torch.cuda.Event"]] = {}
+
+
+def _clear_workspace(ws: torch.Tensor, word: int) -> None:
+    """After a reported failure: empty the partial-sum slots (late slices may have left values in
+    them that later calls would take for ready) and drop the reported bits."""
+    if word & STATUS_SUM_MISSING:
+        ws[WS_HEADER_BYTES:].zero_()
+    ws[:4].zero_()
+
+
+def poll_status(device=None, wait: bool = False) -> None:
+    """The serving path's look at the status words, without a synchronisation of its own: every call
+    evaluates the copy the previous call started (if it has completed, or after waiting for it when
+    `wait` is set) and starts the next one, a 4-byte device-to-host copy into pinned memory on the
+    workspace's stream.  Raises DeltaKernelError / warns as `raise_for_status` says; a reported
+    failure also clears the workspace.  With `wait` the current state is read as well (this
+    synchronises with the workspace's stream)."""
+    idx = None if device is None else torch.device(device).index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    found = 0
+    for key, ws in list(_workspaces.items()):
+        if key[0] != idx:
+            continue
+        stream = torch.cuda.ExternalStream(key[1], device=ws.device) if key[1] else torch.cuda.default_stream(ws.device)
+        pending = _status_polls.pop(key, None)
+        host = pending[0] if pending is not None else torch.zeros(1, dtype=torch.int32, pin_memory=True)
+        word = 0
+        if pending is not None:
+            if wait:
+                pending[1].synchronize()
+            if pending[1].query():
+                word = int(host[0])
+            else:
+                _status_polls[key] = pending          # not in yet: looked at by the next call
+                continue
+        with torch.cuda.stream(stream):
+            if wait:
+                # the state as of now, too
+                host.copy_(ws[:4].view(torch.int32), non_blocking=True)
+                stream.synchronize()
+                word |= int(host[0])
+            if word:
+                _clear_workspace(ws, word)            # before the next copy is started
+            if not wait:
+                ev = torch.cuda.Event()
+                host.copy_(ws[:4].view(torch.int32), non_blocking=True)
+                ev.record()
+                _status_polls[key] = (host, ev)
+        found |= word
+    if found:
+        raise_for_status(found)
 
 
 # ---------------------------------------------------------------------------------------------

@@ -39,18 +39,19 @@ def random_native_stack(K: int, N: int, bits: int, group_size: int, num_deltas: 
 
 
 def gaussian_native_stack(K: int, N: int, bits: int, group_size: int, num_deltas: int, device,
-                          generator: torch.Generator, sigma: float = 1e-3, return_deltas: bool = False):
+                          generator: torch.Generator, sigma: float = 1e-3, keep_deltas=()):
     """(qweight_stacked, meta_stacked, scales_stacked) for `num_deltas` slots, each the compressed
     form of its own delta ~ N(0, sigma) [N, K] fp32 (drawn on the device from `generator`).
-    return_deltas: also the fp32 deltas, as a list (for checks against the CPU restatement)."""
+    keep_deltas: slot numbers whose fp32 delta is returned as well, as a dict slot -> tensor (for
+    checks against the CPU restatement of the compression pipeline)."""
     qs, ms, ss = ops.stacked_shapes(K, N, bits, group_size)
     q = torch.empty((num_deltas,) + qs, dtype=torch.int32, device=device)
     m = torch.empty((num_deltas,) + ms, dtype=torch.int16, device=device)
     s = torch.empty((num_deltas,) + ss, dtype=torch.float16, device=device)
-    deltas = []
+    deltas = {}
     for d in range(num_deltas):
         delta = torch.randn((N, K), device=device, dtype=torch.float32, generator=generator) * sigma
         q[d], m[d], s[d] = ops.compress_delta(delta, bits, group_size)
-        if return_deltas:
-            deltas.append(delta)
-    return (q, m, s, deltas) if return_deltas else (q, m, s)
+        if d in keep_deltas:
+            deltas[d] = delta
+    return (q, m, s, deltas) if keep_deltas else (q, m, s)

@@ -81,6 +81,22 @@ def test_layer_protocol(dev):
         base.weight.copy_(p["wb"])
     assert o.rel_err(out_w2.cpu().numpy(), o.forward_ref(p["x_np"], 2 * p["wb_np"], p["dts"], oracle_ids)) <= TOL
     assert torch.equal(layer(p["x"])[0], out)
+    # the serving engine's way of loading a base weight: the parameter's weight_loader writes
+    # param.data, which moves no version counter; a loader the parameter carried when the layer was
+    # made is wrapped, so the tiles follow
+    lin2 = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.float16)
+    lin2.weight.weight_loader = lambda param, loaded: param.data.copy_(loaded)
+    wrapped = from_layer(lin2, 4, DeltaConfig(max_deltas=4, max_bitwidth=bits), ["gate_proj", "up_proj"])
+    for slot in (1, 2, 3):
+        wrapped.set_delta(slot, bits, layer.qweight_stacked[slot], None, layer.scales_stacked[slot], None, layer.meta_stacked[slot])
+    wrapped.set_mapping(index_buf, None, None, None, [t])
+    lin2.weight.weight_loader(lin2.weight, p["wb"])
+    assert torch.equal(wrapped(p["x"])[0], out)
+    # a write through .data from anywhere else cannot be seen by the layer (documented): the caller
+    # refreshes the tiles
+    lin2.weight.data.mul_(2.0)
+    wrapped.refresh_base_tiles()
+    assert torch.equal(wrapped(p["x"])[0], out_w2)
     # reset a slot: its tokens fall back to the base layer
     layer.reset_delta(2)
     out2, _ = layer(p["x"])

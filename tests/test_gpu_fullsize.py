@@ -1,4 +1,7 @@
-"""Parity at the benchmark's full layer shapes (Llama-2-7B / 13B projections).
+"""Parity at the benchmark's full layer shapes (Llama-2-7B / 13B projections), on the deltas the
+benchmark configurations describe: drawn from N(0, sigma), scales from the un-pruned values, pruned
+2:4 by magnitude, quantised (compressed on the GPU by ops.compress_delta; sampled rows of the result
+are held against the CPU restatement of that pipeline, bit for bit).
 
 The CPU oracle cannot dequantise and multiply whole 4096 x 11008 layers in seconds, so each case is
 checked three ways:
@@ -15,7 +18,7 @@ import torch
 
 from oracle import dz_oracle as o
 from deltazip_amd import ops
-from deltazip_amd.synthetic import random_native_stack
+from deltazip_amd.synthetic import gaussian_native_stack
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-2   # max relative error of fp16 outputs against the fp32 reference (floor 1e-3 * max|ref|)
@@ -70,12 +73,14 @@ def _ids(kind, t, nd, seed):
 @pytest.mark.parametrize("K,N,bits,gs,nd,T,kind", CASES)
 def test_full_size_layer(dev, K, N, bits, gs, nd, T, kind):
     gen = torch.Generator(device=dev).manual_seed(K + N + bits + T)
-    q, m, s = random_native_stack(K, N, bits, gs, nd, dev, gen)
-    wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
-    x = torch.randn((T, K), device=dev, generator=gen).half()
     ids_np = _ids(kind, T, nd, K + T)
     if T > 2:
         ids_np[0] = -1
+    first = int(min(d for d in ids_np if d >= 0))
+    sigma = 2e-3 if T == 1 else 1e-3          # configuration 1 draws its delta from N(0, 2e-3)
+    q, m, s, fp32 = gaussian_native_stack(K, N, bits, gs, nd, dev, gen, sigma, keep_deltas=(first,))
+    wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
+    x = torch.randn((T, K), device=dev, generator=gen).half()
     ids = torch.from_numpy(ids_np).to(dev)
     y = ops.apply_delta(x, q, s, m, ids, wb)
     torch.cuda.synchronize()
@@ -93,6 +98,16 @@ def test_full_size_layer(dev, K, N, bits, gs, nd, T, kind):
         got = ops.dequant(q[d], m[d], s[d], K, N, bits)[torch.from_numpy(rows).to(dev)].cpu().numpy()
         assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), f"dequant differs for slot {d}"
         dts[d] = ref
+        if d in fp32:
+            # the same rows through the CPU restatement of the reference's pipeline (scales from the
+            # un-pruned delta, 2:4 by magnitude, round to nearest, pack, dequantise)
+            rows_d = fp32[d][torch.from_numpy(rows).to(dev)].cpu().numpy()
+            codes_o, sc_o, zeros_o, _ = o.compress_delta(rows_d, bits, gs)
+            qw_o, qz_o, sc16_o, gidx_o = o.pack_codes_gptq(codes_o, zeros_o, sc_o, bits)
+            want = o.dequant_gptq(qw_o, qz_o, sc16_o, gidx_o, bits)        # [K, rows]
+            assert np.array_equal(got.view(np.uint16), np.ascontiguousarray(want.T).view(np.uint16)), \
+                f"compressed delta of slot {d} differs from the CPU pipeline"
+    del fp32
     tok = np.nonzero(np.isin(ids_np, list(dts.keys()) + [-1]))[0][:64]
     xs = x[torch.from_numpy(tok).to(dev)].cpu().numpy().astype(np.float32)
     wbs = wb[torch.from_numpy(rows).to(dev)].cpu().numpy().astype(np.float32)
