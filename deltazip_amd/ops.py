@@ -470,6 +470,8 @@ def poll_status(device=None, wait: bool = False) -> None:
     workspace's stream.  Raises DeltaKernelError / warns as `raise_for_status` says; a reported
     failure also clears the workspace.  With `wait` the current state is read as well (this
     synchronises with the workspace's stream)."""
+    if not _workspaces:
+        return                                        # no fused call has run yet (or no GPU at all)
     idx = None if device is None else torch.device(device).index
     if idx is None:
         idx = torch.cuda.current_device()
