@@ -585,6 +585,27 @@ def main():
                     "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
                     "kernel": "dz_gemm24_kernel", "algorithmic_flops_per_call": step_flops / len(groups),
                     "avg_call_us": round(avg_launch_s * 1e6, 2)}
+        if not args.no_probe:
+            # Yardstick: the library's dense fp16 GEMM (torch.mm -> hipBLASLt / rocBLAS) on the same base
+            # weights and activations, in the step's order over the same resident layers -- the base half
+            # of the work alone, no delta.  The fused kernel issues 1.5 matrix instructions per base one
+            # (a 16x16x64 sparse product for every two dense 16x16x32), so its rate in issued matrix
+            # instructions is 1.5 x its rate in base flops.
+            def lib_step(i):
+                for name, K, N, x, wb, q, m, s, y, _ in layers[i % len(layers)]:
+                    torch.mm(x, wb.t(), out=y)
+            us_lib = time_loop(lib_step, max(4, min(steps, 20)), warm=3)
+            us_own = time_loop(step, max(4, min(steps, 20)), warm=3)
+            lib_tf = step_flops / us_lib / 1e6
+            own_tf = step_flops / us_own / 1e6
+            roofline["practical_peak"] = {
+                "what": "torch.mm (the ROCm GEMM library) on the same base weights and activations: dense fp16 "
+                        "base product only, no delta; both timed back to back the same way",
+                "library_step_us": round(us_lib, 1), "library_tflops": round(lib_tf, 1),
+                "library_frac_of_peak": round(lib_tf / MFMA_F16_PEAK_TFLOPS, 4),
+                "fused_step_us": round(us_own, 1), "fused_base_tflops": round(own_tf, 1),
+                "fused_matrix_instruction_tflops_equivalent": round(1.5 * own_tf, 1) if bits == 2 else None,
+                "fused_over_library": round(us_lib / us_own, 4)}
 
     out = {
         "metric": "multi-delta linear tokens/s + achieved HBM TB/s (% peak), Llama-7B shapes",

@@ -3,9 +3,11 @@
 // for tokens grouped by delta slot (a table of row blocks, each with one slot).
 //
 // One workgroup (8 wavefronts, two per SIMD) computes 256 output features x 256 tokens of one row
-// block; each wavefront owns 128 features x 64 tokens as 8 x 4 tiles of 16 x 16 (128 fp32
+// block; each wavefront owns 64 features x 128 tokens as 4 x 8 tiles of 16 x 16 (128 fp32
 // accumulators, in ordinary vector registers: the sparse instruction does not accumulate in the
-// accumulation registers).  K is walked in slabs of 64 columns; weight slab and activation slab go
+// accumulation registers).  64 features are two n-pairs of the delta: their packed words are
+// unpacked and scaled once per slab and used for all eight token tiles (with 128 features x 64
+// tokens per wavefront the same four n-pairs were unpacked by four wavefronts each).  K is walked in slabs of 64 columns; weight slab and activation slab go
 // from global memory straight into LDS (two buffers, the next slab is on its way while this one is
 // multiplied).  The delta's packed codes and 2-bit positions (native layout: 16 bytes per lane per
 // 32 x 256 tile, already in operand order) are staged in LDS one k-block ahead, read back by the
@@ -51,7 +53,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];   // [2 buffers][w slab | x slab]
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wn = wave & 1, wq = wave >> 1;       // feature half (128), token quarter (64)
+  const int wn = wave & 3, wq = wave >> 2;       // feature quarter (64), token half (128)
   const int li = lane & 15, lg = lane >> 4;
   const uint32_t MAGIC = magic_vgpr();
 
@@ -68,14 +70,14 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   const int nslab1 = P.K / BK;
   const int nb = P.w ? nslab1 : 0, nd = has_delta ? nslab1 : 0, total = nb + nd;
   const unsigned Kb = (unsigned)P.K * 2u;
-  // a wavefront whose 64 token rows lie beyond the block only helps with the loads
-  const bool has_rows = row_lo + wq * 64 < row_hi;
+  // a wavefront whose 128 token rows lie beyond the block only helps with the loads
+  const bool has_rows = row_lo + wq * 128 < row_hi;
 
-  f4_t acc[8][4];
+  f4_t acc[4][8];   // [feature tile][token tile]
 #pragma unroll
-  for (int a = 0; a < 8; ++a)
+  for (int a = 0; a < 4; ++a)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) acc[a][b] = (f4_t){0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < 8; ++b) acc[a][b] = (f4_t){0.f, 0.f, 0.f, 0.f};
 
   // ---- slab loader.  A slab is 32 requests of 1 KiB (8 rows x 128 bytes); every wavefront issues 4
   // of the weight slab and 4 of the activation slab.  Lane l fills LDS row l/8, physical chunk l%8
@@ -147,15 +149,15 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   // scales of scale group gi: lane l fetches the scale of row 32*p + l % 32 of n-pair p (one
   // 2-byte load per n-pair, nothing depends on it until the group starts); the two values a lane
   // multiplies with -- rows i and 16 + i -- reach it by a cross-lane move when the group starts
-  auto load_scales = [&](int (&raw)[4], int gi) {
+  auto load_scales = [&](int (&raw)[2], int gi) {
     const _Float16* sp = P.scales + (size_t)slot * P.scales_slot + (size_t)min(gi, P.G - 1) * P.N;
 #pragma unroll
-    for (int p = 0; p < 4; ++p)
-      raw[p] = *(const unsigned short*)(sp + min(n0 + wn * 128 + 32 * p + (lane & 31), P.N - 1));
+    for (int p = 0; p < 2; ++p)
+      raw[p] = *(const unsigned short*)(sp + min(n0 + wn * 64 + 32 * p + (lane & 31), P.N - 1));
   };
-  auto spread_scales = [&](h2_t (&sc)[4], const int (&raw)[4]) {
+  auto spread_scales = [&](h2_t (&sc)[2], const int (&raw)[2]) {
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < 2; ++p) {
       const unsigned lo = (unsigned)__builtin_amdgcn_ds_bpermute(li << 2, raw[p]) & 0xffffu;
       const unsigned hi = (unsigned)__builtin_amdgcn_ds_bpermute((16 + li) << 2, raw[p]);
       H2U u;
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   int foff[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) foff[h] = (((4 * h + lg) ^ ((li >> 1) & 7)) << 4);
-  const int wrow = (wn * 128 + li) * 128, xrow = (wq * 64 + li) * 128;
+  const int wrow = (wn * 64 + li) * 128, xrow = (wq * 128 + li) * 128;
 
   // The delta pass starts with activation slabs 0 and 1 and the first k-block's packed operands
   // already requested: at the start when there is no base pass, else during the last base slab
@@ -190,8 +192,8 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   constexpr bool FUSE = BITS == 2;   // (two staged k-blocks of 4-bit operands do not fit beside the slab buffers)
   if constexpr (FUSE) {
     const bool do_w = nb > 0, do_d = nd > 0;   // workgroup-uniform
-    h2_t sc[4];
-    int scn[4];
+    h2_t sc[2];
+    int scn[2];
     if (total > 0) issue(0, 0, do_w);
     if (do_d) {
       issue_delta(0, 0);
@@ -204,7 +206,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       __syncthreads();
       if (s + 1 < nslab1) issue(s + 1, buf ^ 1, do_w);
       if (do_d) {
-        // the packed words of k-block kb sit in stage kb & 1 (each lane's words j of its four
+        // the packed words of k-block kb sit in stage kb & 1 (each lane's words j of its two
         // n-pairs are read from there slab by slab); the other stage, last read during k-block
         // kb - 1, takes k-block kb + 1
         if (j == 1 && kb + 1 < P.NKB) issue_delta(kb + 1, (kb + 1) & 1);
@@ -218,47 +220,78 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
       if (!has_rows) continue;
       const unsigned char* wb = smem + buf * (2 * SLAB);
       const unsigned char* xb = wb + SLAB;
-      // the activation operands of both halves stay in registers for the sparse product; the
-      // weight operands are taken four row tiles at a time (the accumulators leave little room)
-      h16_t B[4];
+      // Reads from LDS run ahead of the matrix instructions that use them: the slab's packed delta
+      // words, its weight operands and the first two token tiles are requested at once, the delta
+      // operands are unpacked while those reads are in flight, and every pair of token tiles is
+      // requested before the products of the pair before it are issued.  (With all reads of a
+      // group of tiles followed by all of its products, the eight wavefronts -- in step after the
+      // barrier -- first queue at the LDS together and then at the matrix cores together.)
+      uint32_t mw[2] = {0u, 0u}, cw[2] = {0u, 0u};
+      if (do_d) {
+        const unsigned char* dsrc = dstage + (kb & 1) * (8 * DT) + (wn * 2) * DT + lane * 16 + j * 4;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const h8_t lo = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[0]);
-        const h8_t hi = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[1]);
-        B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
+        for (int p = 0; p < 2; ++p) {
+          mw[p] = *(const uint32_t*)(dsrc + p * DT);
+          cw[p] = *(const uint32_t*)(dsrc + p * DT + 1024);
+        }
       }
+      // (read without a base weight too -- stale bytes that nothing uses: under a branch the
+      // compiler no longer counts these requests when it waits for the packed words before them)
+      h8_t fw[2][4];
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int ah = 0; ah < 2; ++ah) {
-          if (!do_w) break;
-          h8_t fw[4];
+        for (int a = 0; a < 4; ++a) fw[h][a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
+      auto read_pair = [&](h16_t (&B)[2], int tg) {
 #pragma unroll
-          for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + (4 * ah + a) * 16 * 128 + foff[h]);
-#pragma unroll
-          for (int b = 0; b < 4; ++b) {
-            const h8_t fxb = h == 0 ? __builtin_shufflevector(B[b], B[b], 0, 1, 2, 3, 4, 5, 6, 7)
-                                    : __builtin_shufflevector(B[b], B[b], 8, 9, 10, 11, 12, 13, 14, 15);
-#pragma unroll
-            for (int a = 0; a < 4; ++a)
-              acc[4 * ah + a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[a], fxb, acc[4 * ah + a][b], 0, 0, 0);
-          }
-          __builtin_amdgcn_sched_barrier(0);   // one group of weight operands at a time
+        for (int b = 0; b < 2; ++b) {
+          const h8_t lo = *(const h8_t*)(xb + xrow + (2 * tg + b) * 16 * 128 + foff[0]);
+          const h8_t hi = *(const h8_t*)(xb + xrow + (2 * tg + b) * 16 * 128 + foff[1]);
+          B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
         }
-      const unsigned char* dsrc = dstage + (kb & 1) * (8 * DT) + (wn * 4) * DT + lane * 16 + j * 4;
+      };
+      h16_t Bc[2], Bn[2];
+      read_pair(Bc, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      h8_t A0[2], A1[2];
+      if (do_d) {
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        if (!do_d) break;
-        const uint32_t mw = *(const uint32_t*)(dsrc + p * DT);
-        const uint32_t cw0 = *(const uint32_t*)(dsrc + p * DT + 1024);
-        h8_t A0, A1;
-        unpack2(cw0, MAGIC, A0, A1);
-        A0 *= sc[p][0];
-        A1 *= sc[p][1];
+        for (int p = 0; p < 2; ++p) {
+          unpack2(cw[p], MAGIC, A0[p], A1[p]);
+          A0[p] *= sc[p][0];
+          A1[p] *= sc[p][1];
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          acc[2 * p][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B[b], acc[2 * p][b], (int)mw, 0, 0);
-          acc[2 * p + 1][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B[b], acc[2 * p + 1][b], (int)mw, 0, 1);
+      for (int tg = 0; tg < 4; ++tg) {
+        if (tg < 3) read_pair(Bn, tg + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (do_w) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              const h8_t fxb = h == 0 ? __builtin_shufflevector(Bc[b], Bc[b], 0, 1, 2, 3, 4, 5, 6, 7)
+                                      : __builtin_shufflevector(Bc[b], Bc[b], 8, 9, 10, 11, 12, 13, 14, 15);
+#pragma unroll
+              for (int a = 0; a < 4; ++a)
+                acc[a][2 * tg + b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[h][a], fxb, acc[a][2 * tg + b], 0, 0, 0);
+            }
+        }
+        if (do_d) {
+#pragma unroll
+          for (int p = 0; p < 2; ++p)
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+              acc[2 * p][2 * tg + b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0[p], Bc[b], acc[2 * p][2 * tg + b], (int)mw[p], 0, 0);
+              acc[2 * p + 1][2 * tg + b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1[p], Bc[b], acc[2 * p + 1][2 * tg + b], (int)mw[p], 0, 1);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (tg < 3) {
+          Bc[0] = Bn[0];
+          Bc[1] = Bn[1];
         }
       }
     }
@@ -280,23 +313,23 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     const unsigned char* xb = wb + SLAB;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      h8_t fw[8], fx[4];
+      h8_t fw[4], fx[8];
 #pragma unroll
-      for (int a = 0; a < 8; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
+      for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
 #pragma unroll
-      for (int b = 0; b < 4; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[h]);
+      for (int b = 0; b < 8; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[h]);
 #pragma unroll
-      for (int b = 0; b < 4; ++b)
+      for (int b = 0; b < 8; ++b)
 #pragma unroll
-        for (int a = 0; a < 8; ++a)
+        for (int a = 0; a < 4; ++a)
           acc[a][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[a], fx[b], acc[a][b], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);   // one half-slab's operands at a time
     }
   }
   // ---- delta pass
-  Frag<BITS> cur[4];
-  h2_t sc[4];
-  int scn[4];
+  Frag<BITS> cur[2];
+  h2_t sc[2];
+  int scn[2];
   if (nd > 0) load_scales(scn, 0);
   int gi = 0, gleft = P.gslabs;   // current scale group, slabs left in it
   for (int sd = 0; sd < nd; ++sd) {
@@ -317,9 +350,9 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     }
     if (j == 0) {
       // this k-block's packed operands were staged during the previous k-block
-      const unsigned char* dsrc = dstage + (wn * 4) * DT + lane * 16;
+      const unsigned char* dsrc = dstage + (wn * 2) * DT + lane * 16;
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
+      for (int p = 0; p < 2; ++p) {
         cur[p].meta = *(const u4_t*)(dsrc + p * DT);
         cur[p].code[0] = *(const u4_t*)(dsrc + p * DT + 1024);
         if (BITS == 4) cur[p].code[BITS == 2 ? 0 : 1] = *(const u4_t*)(dsrc + p * DT + 2048);
@@ -338,15 +371,10 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     }
     if (!has_rows) continue;
     const unsigned char* xb = smem + (sd & 3) * SLAB;
-    h16_t B[4];
+    h8_t A0[2], A1[2];
+    uint32_t mwp[2];
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const h8_t lo = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[0]);
-      const h8_t hi = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[1]);
-      B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
-    }
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int p = 0; p < 2; ++p) {
       // word j of the lane's four words; a compile-time index after unrolling over the four cases
       uint32_t cw0 = 0, cw1 = 0, mw = 0;
 #pragma unroll
@@ -361,20 +389,32 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
           }
         }
       }
-      h8_t A0, A1;
       if (BITS == 2) {
-        unpack2(cw0, MAGIC, A0, A1);
+        unpack2(cw0, MAGIC, A0[p], A1[p]);
       } else {
-        A0 = unpack4(cw0, MAGIC);
-        A1 = unpack4(cw1, MAGIC);
+        A0[p] = unpack4(cw0, MAGIC);
+        A1[p] = unpack4(cw1, MAGIC);
       }
-      A0 *= sc[p][0];
-      A1 *= sc[p][1];
+      A0[p] *= sc[p][0];
+      A1[p] *= sc[p][1];
+      mwp[p] = mw;
+    }
+#pragma unroll
+    for (int tg = 0; tg < 2; ++tg) {
+      h16_t B[4];
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        acc[2 * p][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0, B[b], acc[2 * p][b], (int)mw, 0, 0);
-        acc[2 * p + 1][b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1, B[b], acc[2 * p + 1][b], (int)mw, 0, 1);
+        const h8_t lo = *(const h8_t*)(xb + xrow + (4 * tg + b) * 16 * 128 + foff[0]);
+        const h8_t hi = *(const h8_t*)(xb + xrow + (4 * tg + b) * 16 * 128 + foff[1]);
+        B[b] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15);
       }
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          acc[2 * p][4 * tg + b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A0[p], B[b], acc[2 * p][4 * tg + b], (int)mwp[p], 0, 0);
+          acc[2 * p + 1][4 * tg + b] = __builtin_amdgcn_smfmac_f32_16x16x64_f16(A1[p], B[b], acc[2 * p + 1][4 * tg + b], (int)mwp[p], 0, 1);
+        }
     }
   }
 
@@ -382,21 +422,21 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
 
   // ---- store: lane (i, g) holds features 4*g .. 4*g + 3 of tile a for token i of tile b
 #pragma unroll
-  for (int b = 0; b < 4; ++b) {
-    const int pos = row_lo + wq * 64 + b * 16 + li;
+  for (int b = 0; b < 8; ++b) {
+    const int pos = row_lo + wq * 128 + b * 16 + li;
     if (pos >= row_hi) continue;
     const int row = P.perm ? P.perm[pos] : pos;
-    _Float16* yrow = P.y + (size_t)row * P.ldy + n0 + wn * 128 + 4 * lg;
-    h4_t old[8];
+    _Float16* yrow = P.y + (size_t)row * P.ldy + n0 + wn * 64 + 4 * lg;
+    h4_t old[4];
     if (P.accumulate) {
-      // all eight reads of the token's row in flight together
+      // all four reads of the token's row in flight together
 #pragma unroll
-      for (int a = 0; a < 8; ++a)
-        old[a] = (n0 + wn * 128 + a * 16 + 4 * lg < P.N) ? *(const h4_t*)(yrow + a * 16) : (h4_t){0, 0, 0, 0};
+      for (int a = 0; a < 4; ++a)
+        old[a] = (n0 + wn * 64 + a * 16 + 4 * lg < P.N) ? *(const h4_t*)(yrow + a * 16) : (h4_t){0, 0, 0, 0};
     }
 #pragma unroll
-    for (int a = 0; a < 8; ++a) {
-      if (n0 + wn * 128 + a * 16 + 4 * lg >= P.N) continue;
+    for (int a = 0; a < 4; ++a) {
+      if (n0 + wn * 64 + a * 16 + 4 * lg >= P.N) continue;
       f4_t v = acc[a][b];
       if (P.accumulate) v += (f4_t){(float)old[a][0], (float)old[a][1], (float)old[a][2], (float)old[a][3]};
       const h4_t o = {(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
