@@ -345,6 +345,12 @@ def main():
     # up to 128 tokens the layer reads its base weight from the tiled copy it makes at creation
     # (dz_tile_base); --row-major-base measures the fused kernel on the plain [N, K] weight instead
     fused = T <= 128
+    if not fused and not args.separate_launches and [sh[0] for sh in shapes] == [sh[0] for sh in SHAPES]:
+        # prefill-sized calls: q/k/v and gate/up are one layer each, with one weight and one stacked delta
+        # over the fused output dimension -- how the merged layers hold and run them
+        # (serving/vllm/delta/layers_marlin.py:281-487)
+        (_, K0, Nq), (_, _, Nk), (_, _, Nv), o, (_, _, Ng), (_, _, Nu), down = shapes
+        shapes = [("q+k+v", K0, Nq + Nk + Nv), o, ("gate+up", K0, Ng + Nu), down]
     tiled_base = fused and not args.row_major_base
     default_workload = (args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
                         and not args.row_major_base)
@@ -424,12 +430,15 @@ def main():
         def call(i, idx):
             launch(i, idx, single)
     else:
-        # prefill-sized: the host wrapper groups the batch and runs the packed-delta GEMM
+        # prefill-sized: the batch is ordered by delta and cut into row blocks once per step (inside the
+        # timed region; as the reference converts its mapping once per batch), then one launch of the
+        # packed-delta GEMM per layer
         order = None
+        blocks = [None]
 
         def call(i, idx):
             name, K, N, x, wb, q, m, s, y, _ = layers[i % len(layers)][idx]
-            ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y)
+            ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y, order=blocks[0])
 
         def launch(i, gi, prep=None):
             call(i, groups[gi][0])
@@ -438,6 +447,8 @@ def main():
         ids_t = ids if ids_t is None else ids_t
 
         def step(i):
+            if not fused:
+                blocks[0] = ops.row_blocks(ids_t, S)
             if fused and order is not None:
                 rc = lib.dz_token_order(C.c_void_p(ids_t.data_ptr()), T, S, C.c_void_p(order.data_ptr()), C.c_void_p(stream))
                 if rc:

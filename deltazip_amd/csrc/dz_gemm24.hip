@@ -45,7 +45,7 @@ struct Gemm24Params {
   const dz_gemm_tile* tiles;     // row blocks (device memory)
   const int* perm;               // token order or nullptr
   _Float16* y;
-  int T, K, N, S, G, gslabs, accumulate, ldy, tiles_m, tiles_n, NKB, NP;   // gslabs: slabs per scale group
+  int T, K, N, S, G, gslabs, accumulate, ldy, tiles_m, tiles_n, NKB, NP, m_first;   // gslabs: slabs per scale group
 };
 
 template <int BITS>
@@ -59,9 +59,13 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
 
   // workgroup -> tile: XCD-local blocks of GM x GN tiles
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
-  const int sbn = (P.tiles_n + GN - 1) / GN;
+  const int sbn = (P.tiles_n + GN - 1) / GN, sbm = (P.tiles_m + GM - 1) / GM;
   const int sb = (q / (GM * GN)) * 8 + xcd, r = q % (GM * GN);
-  const int tm = (sb / sbn) * GM + r / GN, tn = (sb % sbn) * GN + r % GN;
+  // consecutive blocks -- the ones the eight XCDs work on at the same time -- walk the smaller
+  // operand: the larger one is then fetched from memory once, and the smaller one, fetched once per
+  // block row or column, is found in the last-level cache
+  const int sbi = P.m_first ? sb % sbm : sb / sbn, sbj = P.m_first ? sb / sbm : sb % sbn;
+  const int tm = sbi * GM + r / GN, tn = sbj * GN + r % GN;
   if (tm >= P.tiles_m || tn >= P.tiles_n) return;
   const int row_lo = P.tiles[tm].row_lo, row_hi = P.tiles[tm].row_hi, slot = P.tiles[tm].group;
   if (row_hi <= row_lo) return;                  // unused entry of the table
@@ -501,6 +505,7 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   P.tiles_m = ntiles;
   P.tiles_n = (N + BN - 1) / BN;
   const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
+  P.m_first = N > T;   // the weight is the larger operand
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
   // two slab buffers (= four ring stages of the delta pass) + the staged packed operands: one

@@ -70,6 +70,7 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.indices: Optional[torch.Tensor] = None
         self.indices_len: Optional[List[int]] = None
         self.token_order: Optional[torch.Tensor] = None
+        self.row_blocks: Optional[list] = None
 
     # -- state ---------------------------------------------------------------------------------
     def create_delta_weights(self, max_deltas: int, delta_config: DeltaConfig, model_config=None) -> None:
@@ -145,18 +146,23 @@ class LinearWithDelta(BaseLayerWithDelta):
 
     def set_mapping(self, base_indices: torch.Tensor, sampler_indices=None, sampler_indices_padded=None,
                     embeddings_indices=None, indices_len: Optional[List[int]] = None,
-                    token_order: Optional[torch.Tensor] = None):
+                    token_order: Optional[torch.Tensor] = None, row_blocks: Optional[list] = None):
         # a view of the manager's buffer, re-read on the device at every call
         self.indices = base_indices
         self.indices_len = indices_len if indices_len is not None else [base_indices.numel()]
         # optional: the manager's buffer with the order in which the kernel takes the tokens of a
         # 33..128-token batch (the manager refreshes it with the mapping; None: computed per call)
         self.token_order = token_order
+        # optional: the manager's one-element list holding ops.row_blocks() of the current batch when
+        # it has more than 128 tokens (None inside: made per call)
+        self.row_blocks = row_blocks
 
     # -- compute -------------------------------------------------------------------------------
     def apply_weights(self, x: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
         T = self.indices_len[0]
         order = self.token_order[:T] if self.token_order is not None and 32 < T <= ops.MAX_TOKENS_FUSED else None
+        if T > ops.MAX_TOKENS_FUSED and self.row_blocks is not None:
+            order = self.row_blocks[0]
         w = self.base_layer.weight
         if self.base_tiled is not None and self._tiled_of != (w.data_ptr(), w._version):
             self.refresh_base_tiles()

@@ -122,6 +122,9 @@ class DeltaModelManager:
         # order in which the fused kernel takes the tokens of a 33..128-token batch; refreshed with
         # the mapping, shared by every linear layer
         self.token_order = torch.zeros(ops.MAX_TOKENS_FUSED, dtype=torch.int32, device=self.device)
+        # larger batches: the tokens ordered by delta and cut into row blocks, made once per batch
+        # (the layers keep a reference to this list)
+        self.row_blocks = [None]
         # raw delta ids of the batch ([tokens | sampled rows]) and the id resident in each slot:
         # staged in pinned host memory, copied with one transfer each
         pin = self.device.type == "cuda"
@@ -264,6 +267,9 @@ class DeltaModelManager:
                     self.embeddings_indices)
         if 32 < T <= ops.MAX_TOKENS_FUSED:
             ops.token_order(self.base_indices[:T], self.delta_slots, out=self.token_order)
+        self.row_blocks[0] = None
+        if T > ops.MAX_TOKENS_FUSED and not ops.takes_fused_chunks(T, self.delta_slots):
+            self.row_blocks[0] = ops.row_blocks(self.base_indices[:T], self.delta_slots)
         # the layers keep a reference to this list
         self.indices_len[:] = (T, P, P, T)
 
@@ -313,7 +319,8 @@ class DeltaModelManager:
             self._register_packed_modules(module_name)
             if isinstance(new_module, LinearWithDelta):
                 new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
-                                       self.embeddings_indices, self.indices_len, token_order=self.token_order)
+                                       self.embeddings_indices, self.indices_len, token_order=self.token_order,
+                                       row_blocks=self.row_blocks)
             else:
                 new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
                                        self.embeddings_indices, self.indices_len)

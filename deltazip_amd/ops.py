@@ -158,6 +158,31 @@ def segment(indices: torch.Tensor, num_slots: int):
     return perm, off
 
 
+class RowBlocks:
+    """A batch of more than 128 tokens ordered by delta id and cut into row blocks of one delta each
+    (what dz_segment and dz_build_tiles write): depends on the indices only, so it can be made once
+    per batch and passed to every layer call of the step (`order=`)."""
+    __slots__ = ("perm", "tiles", "max_tiles", "T", "S")
+
+    def __init__(self, perm, tiles, max_tiles, T, S):
+        self.perm, self.tiles, self.max_tiles, self.T, self.S = perm, tiles, max_tiles, T, S
+
+
+def row_blocks(indices: torch.Tensor, num_slots: int) -> RowBlocks:
+    """Row blocks of a prefill-sized batch, as the reference converts its mapping once per batch
+    (serving/vllm/delta/models.py:421-435).  Two small launches, nothing read back to the host."""
+    indices = indices.reshape(-1)
+    if not indices.is_contiguous():
+        raise ValueError("indices must be contiguous")
+    T = indices.numel()
+    perm, seg_off = segment(indices, num_slots)
+    max_tiles = (T + 255) // 256 + min(num_slots + 1, T)
+    tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=indices.device)
+    _lib.check(_lib.lib().dz_build_tiles(seg_off.data_ptr(), num_slots, tiles.data_ptr(), max_tiles, _stream()),
+               "dz_build_tiles")
+    return RowBlocks(perm, tiles, max_tiles, T, num_slots)
+
+
 def apply_delta_embed(x: torch.Tensor, delta_weights: torch.Tensor, indices: torch.Tensor,
                       base_weight: torch.Tensor) -> torch.Tensor:
     """Embedding lookup where every token reads the table of its own delta
@@ -560,8 +585,9 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
                        order: Optional[torch.Tensor] = None,
                        base_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """y = x @ W_base^T + x @ dequant(delta[indices])^T.  `out` may be a column slice of a wider
-    tensor (last-dim stride 1); with accumulate=True the result is added to it.  `order`: the
-    result of `token_order(indices, S)` when the caller already has it for this batch.
+    tensor (last-dim stride 1); with accumulate=True the result is added to it.  `order`: what the
+    caller already has for this batch -- the result of `token_order(indices, S)` (up to 128
+    tokens) or of `row_blocks(indices, S)` (more).
     `base_tiled`: `tile_base(base_weight)`, read instead of the row-major weight by calls of up to
     128 tokens (the results are the same bit for bit)."""
     _need_cuda(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices)
@@ -608,8 +634,11 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
                                    out=out[r:r + MAX_TOKENS_FUSED], accumulate=accumulate, base_tiled=base_tiled)
             return out
         from .prefill import multi_delta_linear_prefill
+        blocks = order if isinstance(order, RowBlocks) else None
+        if blocks is not None and (blocks.T != T or blocks.S != S):
+            raise ValueError("row blocks were made for another batch size or number of slots")
         return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
-                                          indices, bits=bits, out=out, accumulate=accumulate)
+                                          indices, bits=bits, out=out, accumulate=accumulate, blocks=blocks)
     ws = _workspace(x.device, T, K, N)
     optr = _order_ptr(order, T, x.device)
     if base_tiled is not None:
@@ -661,6 +690,8 @@ def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: 
 
 
 def _order_ptr(order: Optional[torch.Tensor], T: int, device) -> Optional[int]:
+    if isinstance(order, RowBlocks):
+        raise ValueError("row blocks are for batches above %d tokens; pass token_order() here" % MAX_TOKENS_FUSED)
     if order is None or T <= 32:
         return None
     if (not order.is_cuda or order.device != device or order.dtype != torch.int32 or order.numel() < T

@@ -35,12 +35,13 @@ def gemm_f16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
 
 
 def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices,
-                               *, bits: int, out: torch.Tensor, accumulate: bool) -> torch.Tensor:
+                               *, bits: int, out: torch.Tensor, accumulate: bool, blocks=None) -> torch.Tensor:
     """T > 128: tokens are ordered by delta id on the device (dz_segment), the order is cut into
     row blocks of one delta each (dz_build_tiles) and one launch of dz_multi_delta_gemm multiplies
     every block by the base weight and by its delta in packed form.  Nothing is read back to the
-    host, gathered, scattered or dequantised to memory."""
-    from .ops import segment
+    host, gathered, scattered or dequantised to memory.  `blocks`: ops.row_blocks(indices, S) when
+    the caller made it once for the batch (else made here, per call)."""
+    from .ops import row_blocks
     T, K = x2.shape
     N = scales_stacked.shape[-1]
     S = qweight_stacked.shape[0]
@@ -57,13 +58,11 @@ def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked,
         return out
     lib = _lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
-    perm, seg_off = segment(indices, S)
-    max_tiles = (T + 255) // 256 + min(S + 1, T)
-    tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=x2.device)
-    _lib.check(lib.dz_build_tiles(seg_off.data_ptr(), S, tiles.data_ptr(), max_tiles, stream), "dz_build_tiles")
+    if blocks is None:
+        blocks = row_blocks(indices, S)
     rc = lib.dz_multi_delta_gemm(x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
                                  qweight_stacked.data_ptr(), meta_stacked.data_ptr(), scales_stacked.data_ptr(),
-                                 S, bits, group_size, tiles.data_ptr(), max_tiles, perm.data_ptr(),
+                                 S, bits, group_size, blocks.tiles.data_ptr(), blocks.max_tiles, blocks.perm.data_ptr(),
                                  out.data_ptr(), T, K, N, 1 if accumulate else 0, out.stride(0), stream)
     _lib.check(rc, "dz_multi_delta_gemm")
     return out

@@ -274,6 +274,25 @@ def test_prefill_sized_call(dev, kind):
     assert o.rel_err(y, ref) <= TOL
 
 
+def test_row_blocks_made_once_per_batch(dev):
+    """ops.row_blocks(indices, S) made once and passed as `order` to several calls gives, bit for
+    bit, what each call gives when it orders the batch itself; blocks of another batch are refused."""
+    p = make_problem(256, 1024, 2, -1, 4, 700, "uniform", 5, dev)
+    blocks = ops.row_blocks(p["ids"], 4)
+    assert blocks.T == 700 and blocks.S == 4 and blocks.perm.dtype == torch.int32
+    y0 = run_layer(p)
+    for _ in range(2):
+        y1 = ops.multi_delta_linear(p["x"], p["wb"], p["q"], p["s"], p["m"], p["ids"], bits=2, order=blocks)
+        torch.cuda.synchronize()
+        assert torch.equal(y0, y1)
+    with pytest.raises(ValueError):
+        ops.multi_delta_linear(p["x"][:600], p["wb"], p["q"], p["s"], p["m"], p["ids"][:600].contiguous(), bits=2,
+                               order=blocks)
+    with pytest.raises(ValueError):
+        ops.multi_delta_linear(p["x"][:64], p["wb"], p["q"], p["s"], p["m"], p["ids"][:64].contiguous(), bits=2,
+                               order=blocks)
+
+
 @pytest.mark.parametrize("t,nd", [(129, 3), (256, 40), (300, 4), (512, 17)])
 def test_mid_size_batches_go_through_the_fused_kernel_in_chunks(dev, t, nd):
     """Between 129 tokens and a few hundred the matrix-core kernel would leave most of the GPU idle:

@@ -13,6 +13,7 @@ from deltazip_amd.layers import (MergedQKVParallelLinearWithDelta, MergedColumnP
                                  RowParallelLinearWithDelta, VocabParallelEmbeddingWithDelta,
                                  LogitsProcessorWithDelta)
 from deltazip_amd.manager import LRUCache
+from deltazip_amd import ops
 
 H, I, V = 256, 512, 64
 
@@ -391,3 +392,38 @@ def test_checkpoint_to_manager_to_forward(dev):
     before = mgr._staged
     mgr.set_delta_mapping(DeltaMapping((11, 0), (11,)))
     assert mgr._last_mapping == m and mgr._staged is before
+
+
+@pytest.mark.gpu
+def test_manager_makes_row_blocks_once_for_a_large_batch(dev):
+    """A batch above the fused kernel's sizes: the manager orders the tokens by delta and cuts the row
+    blocks once, with the mapping, and every layer call of the step uses them; a smaller batch
+    afterwards drops them again."""
+    bits = 4
+    model = ToyModel(dev)
+    base = {n: m.weight.detach().cpu().numpy().copy() for n, m in model.named_modules() if isinstance(m, nn.Linear)}
+    mgr = create_delta_manager(model, 8, 1024, V, DeltaConfig(max_deltas=3, max_bitwidth=bits, max_cpu_deltas=4),
+                               delta_manager_cls=LRUCacheDeltaModelManager)
+    fused = {}
+    for did in (11, 12):
+        dm, fused[did] = make_delta_model(did, bits, 100 * did)
+        mgr.add_delta(dm)
+        mgr.activate_delta(did)
+    rng = np.random.default_rng(5)
+    ids = tuple(int(i) for i in rng.choice([0, 11, 12], size=600))
+    assert not ops.takes_fused_chunks(len(ids), mgr.delta_slots)
+    mgr.set_delta_mapping(DeltaMapping(ids, ids[:2]))
+    blocks = mgr.row_blocks[0]
+    assert isinstance(blocks, ops.RowBlocks) and blocks.T == 600
+    x = torch.from_numpy(o.make_x(len(ids), H, 3)).to(dev)
+    for name in ("self_attn.qkv_proj", "mlp.gate_up_proj"):
+        layer = model.get_submodule("model.layers.0." + name)
+        assert layer.row_blocks is mgr.row_blocks
+        y, _ = layer(x)
+        torch.cuda.synchronize()
+        ref = o.forward_ref(x.cpu().numpy(), base["model.layers.0." + name], [fused[11][name], fused[12][name]],
+                            np.array([{0: -1, 11: 0, 12: 1}[i] for i in ids]))
+        assert o.rel_err(y.float().cpu().numpy(), ref) <= 1e-2, name
+    assert mgr.row_blocks[0] is blocks          # made once, not per layer call
+    mgr.set_delta_mapping(DeltaMapping(ids[:9], ids[:2]))
+    assert mgr.row_blocks[0] is None
