@@ -304,8 +304,7 @@ def main():
                                                        "(--config 5: decoder layers of the model, default 32)")
     ap.add_argument("--unsorted", action="store_true", help="do not sort the batch by delta id")
     ap.add_argument("--row-major-base", action="store_true",
-                    help="up to 128 tokens: read the base weight as the plain [N, K] tensor instead of the tiled copy "
-                         "a layer makes of it")
+                    help="read the base weight as the plain [N, K] tensor instead of the tiled copy a layer makes of it")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--random-bits", action="store_true",
                     help="fill the delta slots with uniformly random code and position bits instead of compressing "
@@ -351,7 +350,7 @@ def main():
         # (serving/vllm/delta/layers_marlin.py:281-487)
         (_, K0, Nq), (_, _, Nk), (_, _, Nv), o, (_, _, Ng), (_, _, Nu), down = shapes
         shapes = [("q+k+v", K0, Nq + Nk + Nv), o, ("gate+up", K0, Ng + Nu), down]
-    tiled_base = fused and not args.row_major_base
+    tiled_base = not args.row_major_base
     default_workload = (args.config == 2 and not args.unsorted and args.ksplit == 0 and not args.separate_launches
                         and not args.row_major_base)
     ids = make_ids(cfg["ids"], T, S, dev, gen, not args.unsorted)
@@ -369,7 +368,7 @@ def main():
                 dgen = torch.Generator(device=dev).manual_seed(1000 * args.config + 100 * li + si)
                 q, m, s = gaussian_native_stack(K, N, bits, gs, S, dev, dgen, sigma)
             wb = (torch.randn((N, K), device=dev, generator=gen) * 0.02).half()
-            wbt = ops.tile_base(wb) if fused else None     # as a layer does once when it is created
+            wbt = ops.tile_base(wb) if (fused or tiled_base) else None     # as a layer does once when it is created
             if fused and not default_workload:
                 # only one form is read in this run (the default workload also times the other one)
                 if tiled_base:
@@ -437,8 +436,9 @@ def main():
         blocks = [None]
 
         def call(i, idx):
-            name, K, N, x, wb, q, m, s, y, _ = layers[i % len(layers)][idx]
-            ops.multi_delta_linear(x, wb, q, s, m, ids, bits=bits, out=y, order=blocks[0])
+            name, K, N, x, wb, q, m, s, y, wbt = layers[i % len(layers)][idx]
+            ops.multi_delta_linear(x, None if tiled_base else wb, q, s, m, ids, bits=bits, out=y, order=blocks[0],
+                                   base_tiled=wbt if tiled_base else None)
 
         def launch(i, gi, prep=None):
             call(i, groups[gi][0])

@@ -26,6 +26,7 @@ SIGNATURES = {
     "dz_embedding_select": (_i, [_vp, _vp, _vp, _vp, C.c_longlong, _i, _vp, _i, _i, _i, _i, _vp]),
     "dz_build_tiles": (_i, [_vp, _i, _vp, _i, _vp]),
     "dz_multi_delta_gemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
+    "dz_multi_delta_gemm_tiled": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_compress_2of4": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "dz_quant_scales": (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "dz_quant_scales_mse": (_i, [_vp, _i, _i, _i, _i, C.c_float, _i, C.c_float, _vp, _vp, _vp]),

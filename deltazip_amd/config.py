@@ -29,12 +29,19 @@ class DeltaConfig:
     # streams fastest (calls of up to 128 tokens read it, larger ones the row-major weight); off:
     # the base weight is held once and read row-major by every call
     tile_base_weights: bool = True
+    # off (needs tile_base_weights): once the tiled copy is made the layer frees the row-major base
+    # weight -- `base_layer.weight` becomes an empty tensor -- and serves every batch size from the
+    # tiles: one copy of the base model in memory instead of two.  The parameter's weight_loader
+    # still works (the row-major form is rebuilt for the load and dropped again).
+    keep_row_major_base: bool = True
 
     def __post_init__(self):
         if self.max_cpu_deltas is None:
             self.max_cpu_deltas = self.max_deltas
         elif self.max_cpu_deltas < self.max_deltas:
             raise ValueError("max_cpu_deltas must be greater than max_deltas")
+        if not self.keep_row_major_base and not self.tile_base_weights:
+            raise ValueError("keep_row_major_base=False needs tile_base_weights=True")
         if self.max_bitwidth not in (2, 4):
             raise ValueError("max_bitwidth must be 2 or 4")
         if self.group_size != -1 and (self.group_size <= 0 or self.group_size % 64):

@@ -37,7 +37,7 @@ constexpr int GM = 4, GN = 8;             // tiles per XCD block
 
 struct Gemm24Params {
   const _Float16* x;
-  const _Float16* w;             // base weight [N, K] or nullptr
+  const _Float16* w;             // base weight: [N, K], or in tiles (w_tiled), or nullptr
   const u4_t* codes;
   const u4_t* meta;
   const _Float16* scales;
@@ -45,7 +45,7 @@ struct Gemm24Params {
   const dz_gemm_tile* tiles;     // row blocks (device memory)
   const int* perm;               // token order or nullptr
   _Float16* y;
-  int T, K, N, S, G, gslabs, accumulate, ldy, tiles_m, tiles_n, NKB, NP, m_first;   // gslabs: slabs per scale group
+  int T, K, N, S, G, gslabs, accumulate, ldy, tiles_m, tiles_n, NKB, NP, m_first, w_tiled;   // gslabs: slabs per scale group
 };
 
 template <int BITS>
@@ -94,6 +94,14 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     const int R = (wave * 4 + i) * 8 + lr;
     const int lc = (lane & 7) ^ ((R >> 1) & 7);
     goff_w[i] = (unsigned)min(n0 + R, P.N - 1) * Kb + (unsigned)lc * 16u;     // clamped rows: never stored
+    if (P.w_tiled) {
+      // Base weight in tiles: request f = 4 * wave + i is the 1 KiB fragment (feature tile f / 2,
+      // half f % 2) of the slab, contiguous in memory and already in lane order; it lands at the
+      // same place of the slab buffer.  (n-pairs beyond N repeat the last one: never stored.)
+      const int f = wave * 4 + i;
+      const int np = min(n0 / DZ_NPAIR + (f >> 2), P.NP - 1);
+      goff_w[i] = ((unsigned)np * (unsigned)P.NKB * 16u + (unsigned)(((f >> 1) & 1) * 8 + (f & 1))) * 1024u + (unsigned)lane * 16u;
+    }
     const int pos = min(row_lo + R, row_hi - 1);
     const int row = P.perm ? P.perm[pos] : pos;
     goff_x[i] = (unsigned)row * Kb + (unsigned)lc * 16u;
@@ -105,12 +113,13 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
   // base pass: slab s -> buffer s & 1, [weight slab | activation slab]
   auto issue = [&](int s, int buf, bool with_w = true) {
     const int soff = s * (BK * 2);
+    const int soff_w = P.w_tiled ? (s >> 2) * 16384 + (s & 3) * 2048 : soff;   // tile of the k-block, fragments of step s % 4
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       unsigned char* dst = smem + buf * (2 * SLAB) + (wave * 4 + i) * 1024;
       if (with_w)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, (__attribute__((address_space(3))) void*)dst, 16,
-                                                 (int)goff_w[i], soff, 0, 0);
+                                                 (int)goff_w[i], soff_w, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (__attribute__((address_space(3))) void*)(dst + SLAB), 16,
                                                (int)goff_x[i], soff, 0, 0);
     }
@@ -177,6 +186,14 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
 #pragma unroll
   for (int h = 0; h < 2; ++h) foff[h] = (((4 * h + lg) ^ ((li >> 1) & 7)) << 4);
   const int wrow = (wn * 64 + li) * 128, xrow = (wq * 128 + li) * 128;
+  // weight operand of half h, feature tile a: woff[h] + a * 2048 into the weight slab.  From
+  // fragments the lane takes the same columns 32*h + 8*g .. as from the row-major slab: they sit
+  // in fragment g % 2 at lane position 16 * (2*h + g/2) + i (a fragment holds columns
+  // 16*g' + 8*h' + e at position 16*g' + i), so the sums are the same whichever form is read.
+  int woff[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    woff[h] = P.w_tiled ? wn * 8192 + (lg & 1) * 1024 + ((2 * h + (lg >> 1)) * 16 + li) * 16 : wrow + foff[h];
 
   // The delta pass starts with activation slabs 0 and 1 and the first k-block's packed operands
   // already requested: at the start when there is no base pass, else during the last base slab
@@ -245,7 +262,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
 #pragma unroll
       for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int a = 0; a < 4; ++a) fw[h][a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
+        for (int a = 0; a < 4; ++a) fw[h][a] = *(const h8_t*)(wb + woff[h] + a * 2048);
       auto read_pair = [&](h16_t (&B)[2], int tg) {
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
@@ -319,7 +336,7 @@ __global__ __launch_bounds__(512, 2) void dz_gemm24_kernel(const Gemm24Params P)
     for (int h = 0; h < 2; ++h) {
       h8_t fw[4], fx[8];
 #pragma unroll
-      for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 16 * 128 + foff[h]);
+      for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + woff[h] + a * 2048);
 #pragma unroll
       for (int b = 0; b < 8; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 16 * 128 + foff[h]);
 #pragma unroll
@@ -479,10 +496,10 @@ extern "C" int dz_build_tiles(const int32_t* seg_off, int S, dz_gemm_tile* tiles
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
 }
 
-extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
-                                   const void* meta_stacked, const void* scales_stacked, int S, int bits,
-                                   int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
-                                   uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
+static int multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, bool w_tiled, const void* codes_stacked,
+                            const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                            int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                            uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
   if (!x || !y || !tiles || ntiles < 1 || S < 0) return DZ_EINVAL;
   if (S > 0 && (!codes_stacked || !meta_stacked || !scales_stacked)) return DZ_EINVAL;
   size_t cb, mb, sb;
@@ -506,6 +523,7 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   P.tiles_n = (N + BN - 1) / BN;
   const int sbm = (P.tiles_m + GM - 1) / GM, sbn = (P.tiles_n + GN - 1) / GN;
   P.m_first = N > T;   // the weight is the larger operand
+  P.w_tiled = (w_tiled && w_base) ? 1 : 0;
   const int nsb = (sbm * sbn + 7) / 8 * 8;
   const unsigned grid = (unsigned)nsb * GM * GN;
   // two slab buffers (= four ring stages of the delta pass) + the staged packed operands: one
@@ -520,4 +538,21 @@ extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, co
   rc = bits == 2 ? go(dz_gemm24_kernel<2>, 0) : go(dz_gemm24_kernel<4>, 1);
   if (rc) return rc;
   return hipGetLastError() == hipSuccess ? DZ_OK : DZ_ELAUNCH;
+}
+
+extern "C" int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* codes_stacked,
+                                   const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                                   int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                                   uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
+  return multi_delta_gemm(x, w_base, false, codes_stacked, meta_stacked, scales_stacked, S, bits, group_size, tiles,
+                          ntiles, perm, y, T, K, N, accumulate, ldy, stream);
+}
+
+extern "C" int dz_multi_delta_gemm_tiled(const uint16_t* x, const uint16_t* w_base_tiled, const void* codes_stacked,
+                                         const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                                         int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                                         uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
+  if (!w_base_tiled) return DZ_EINVAL;
+  return multi_delta_gemm(x, w_base_tiled, true, codes_stacked, meta_stacked, scales_stacked, S, bits, group_size,
+                          tiles, ntiles, perm, y, T, K, N, accumulate, ldy, stream);
 }

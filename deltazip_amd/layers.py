@@ -87,6 +87,8 @@ class LinearWithDelta(BaseLayerWithDelta):
         self.meta_stacked = torch.zeros((max_deltas,) + ms, dtype=torch.int16, device=w.device)
         self.scales_stacked = torch.zeros((max_deltas,) + ss, dtype=torch.float16, device=w.device)
         self._tile_base = bool(delta_config.tile_base_weights) and w.is_cuda
+        self._drop_row_major = self._tile_base and not delta_config.keep_row_major_base
+        self._row_major_dropped = False
         self.base_tiled = None
         self.refresh_base_tiles()
         self._wrap_weight_loader()
@@ -100,11 +102,24 @@ class LinearWithDelta(BaseLayerWithDelta):
         (model_executor/layers/linear.py:231, 305, 442, 616).  A write that bypasses all three --
         `weight.data.copy_()` from user code leaves the version counter where it was -- cannot be seen
         from here: call this method after it (or `DeltaModelManager.refresh_base_weights()`)."""
-        if not self._tile_base:
+        if not self._tile_base or self._row_major_dropped:
             return
         w = self.base_layer.weight
         self.base_tiled = ops.tile_base(w.detach().contiguous())
         self._tiled_of = (w.data_ptr(), w._version)
+        if self._drop_row_major:
+            # one copy of the base weight: the tiles.  The parameter stays (empty) so that the
+            # module tree and the loader hooks keep their shape.
+            w.data = torch.empty(0, dtype=w.dtype, device=w.device)
+            self._row_major_dropped = True
+
+    def restore_row_major_base(self) -> torch.Tensor:
+        """Rebuilds `base_layer.weight` from the tiled copy (keep_row_major_base=False frees it);
+        `refresh_base_tiles()` afterwards tiles and frees it again."""
+        if self._row_major_dropped:
+            self.base_layer.weight.data = ops.untile_base(self.base_tiled)
+            self._row_major_dropped = False
+        return self.base_layer.weight
 
     def _wrap_weight_loader(self) -> None:
         """The engine's loaders write `param.data` (no version bump): a loader that a base parameter
@@ -115,6 +130,7 @@ class LinearWithDelta(BaseLayerWithDelta):
             return
 
         def weight_loader(*args, **kwargs):
+            self.restore_row_major_base()
             out = loader(*args, **kwargs)
             self.refresh_base_tiles()
             return out
@@ -164,10 +180,13 @@ class LinearWithDelta(BaseLayerWithDelta):
         if T > ops.MAX_TOKENS_FUSED and self.row_blocks is not None:
             order = self.row_blocks[0]
         w = self.base_layer.weight
-        if self.base_tiled is not None and self._tiled_of != (w.data_ptr(), w._version):
+        if self._row_major_dropped:
+            w = None
+        elif self.base_tiled is not None and self._tiled_of != (w.data_ptr(), w._version):
             self.refresh_base_tiles()
+            w = None if self._row_major_dropped else w
         return ops.apply_delta(x, self.qweight_stacked, self.scales_stacked, self.meta_stacked,
-                               self.indices[:T], self.base_layer.weight, order=order, base_tiled=self.base_tiled)
+                               self.indices[:T], w, order=order, base_tiled=self.base_tiled)
 
     def forward(self, input_):
         skip_bias_add = getattr(self.base_layer, "skip_bias_add", False)

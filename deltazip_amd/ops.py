@@ -550,8 +550,8 @@ def _infer(qweight_stacked, scales_stacked, N: int):
 def tile_base(weight: torch.Tensor) -> torch.Tensor:
     """The base weight [N, K] in the tiled form the fused kernel streams fastest (`dz_tile_base`):
     a tensor of the same shape and dtype whose bytes are the tiles.  A layer converts its base
-    weight once and hands both forms to `multi_delta_linear` / `apply_delta_batch` (`base_tiled=`);
-    calls of up to 128 tokens read the tiles, larger ones the row-major weight."""
+    weight once and hands it to `multi_delta_linear` / `apply_delta_batch` (`base_tiled=`); calls of
+    every size read the tiles when they are given."""
     _need_cuda(weight)
     if weight.dtype != torch.float16 or weight.dim() != 2 or not weight.is_contiguous():
         raise ValueError("weight must be a contiguous float16 [N, K] tensor")
@@ -561,10 +561,24 @@ def tile_base(weight: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def _check_tiled(base_tiled, base_weight) -> None:
-    if base_weight is None or base_tiled.shape != base_weight.shape or base_tiled.dtype != torch.float16 \
-            or not base_tiled.is_contiguous() or base_tiled.device != base_weight.device:
-        raise ValueError("base_tiled must be tile_base(base_weight)")
+def untile_base(tiled: torch.Tensor) -> torch.Tensor:
+    """Inverse of `tile_base`: the row-major [N, K] weight from its tiles (plain tensor ops; not on
+    any hot path).  Tile (np, kb) holds fragments (s, j, h); position 16*g + i of a fragment holds
+    W[32*np + 16*s + i][256*kb + 64*j + 16*g + 8*h + e], e = 0..7."""
+    if tiled.dtype != torch.float16 or tiled.dim() != 2 or not tiled.is_contiguous():
+        raise ValueError("tiled must be a contiguous float16 [N, K] tensor")
+    N, K = tiled.shape
+    if N % 32 or K % 256:
+        raise ValueError("N must be a multiple of 32 and K of 256")
+    t = tiled.view(N // 32, K // 256, 2, 4, 2, 4, 16, 8)          # np kb s j h g i e
+    return t.permute(0, 2, 6, 1, 3, 5, 4, 7).reshape(N, K).contiguous()   # np s i | kb j g h e
+
+
+def _check_tiled(base_tiled, base_weight, N: int, K: int, device) -> None:
+    if tuple(base_tiled.shape) != (N, K) or base_tiled.dtype != torch.float16 \
+            or not base_tiled.is_contiguous() or base_tiled.device != device \
+            or (base_weight is not None and base_weight.numel() and base_tiled.shape != base_weight.shape):
+        raise ValueError("base_tiled must be tile_base(base_weight): float16 [N, K], contiguous, on x's device")
 
 
 def takes_fused_chunks(T: int, S: int) -> bool:
@@ -588,8 +602,8 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
     tensor (last-dim stride 1); with accumulate=True the result is added to it.  `order`: what the
     caller already has for this batch -- the result of `token_order(indices, S)` (up to 128
     tokens) or of `row_blocks(indices, S)` (more).
-    `base_tiled`: `tile_base(base_weight)`, read instead of the row-major weight by calls of up to
-    128 tokens (the results are the same bit for bit)."""
+    `base_tiled`: `tile_base(base_weight)`, read instead of the row-major weight (the results are
+    the same bit for bit); base_weight may then be None -- a layer that keeps only the tiled copy."""
     _need_cuda(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices)
     if x.dtype != torch.float16:
         raise ValueError("x must be float16")
@@ -607,6 +621,10 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
         raise ValueError("indices must be a contiguous vector with one entry per token")
     S = qweight_stacked.shape[0]
     N = scales_stacked.shape[-1]
+    if base_tiled is not None:
+        _check_tiled(base_tiled, base_weight, N, K, x.device)
+        if base_weight is not None and base_weight.numel() == 0:
+            base_weight = None
     if base_weight is not None:
         if base_weight.dtype != torch.float16 or tuple(base_weight.shape) != (N, K) or not base_weight.is_contiguous():
             raise ValueError("base_weight must be a contiguous float16 [N, K] tensor")
@@ -638,11 +656,11 @@ def multi_delta_linear(x: torch.Tensor, base_weight: Optional[torch.Tensor], qwe
         if blocks is not None and (blocks.T != T or blocks.S != S):
             raise ValueError("row blocks were made for another batch size or number of slots")
         return multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked,
-                                          indices, bits=bits, out=out, accumulate=accumulate, blocks=blocks)
+                                          indices, bits=bits, out=out, accumulate=accumulate, blocks=blocks,
+                                          base_tiled=base_tiled)
     ws = _workspace(x.device, T, K, N)
     optr = _order_ptr(order, T, x.device)
     if base_tiled is not None:
-        _check_tiled(base_tiled, base_weight)
         one = lambda p: (C.c_void_p * 1)(p)
         rc = _lib.lib().dz_multi_delta_linear_batch_tiled(
             1, one(x2.data_ptr()), one(base_tiled.data_ptr()), one(qweight_stacked.data_ptr()),
@@ -682,7 +700,7 @@ def apply_delta(x: torch.Tensor, qweight_stacked: torch.Tensor, scales_stacked: 
     """Drop-in for serving/vllm/delta/deltazip_marlin.py:10-19.  Returns a new [T, N] tensor;
     indices == -1 selects the base weight only.  (`order`: optional, see `token_order`; `base_tiled`:
     optional, see `tile_base`.)"""
-    N, K = base_weight.shape
+    N, K = base_tiled.shape if base_tiled is not None else base_weight.shape
     bits = _bits_from_shapes(qweight_stacked, K, N)
     y = multi_delta_linear(x, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices, bits=bits,
                            order=order, base_tiled=base_tiled)
@@ -749,7 +767,7 @@ def apply_delta_batch(x, qweight_stacked: Sequence[torch.Tensor], scales_stacked
         if len(base_tiled) != n:
             raise ValueError("one tiled base weight per projection")
         for j in range(n):
-            _check_tiled(base_tiled[j], base_weight[j])
+            _check_tiled(base_tiled[j], base_weight[j], Ns[j], K, x2s[j].device)
         entry, bases = _lib.lib().dz_multi_delta_linear_batch_tiled, base_tiled
     rc = entry(
         n, ptrs(x2s), ptrs(bases), ptrs(qweight_stacked), ptrs(meta_stacked), ptrs(scales_stacked),

@@ -35,12 +35,14 @@ def gemm_f16(x: torch.Tensor, w: torch.Tensor, out: Optional[torch.Tensor] = Non
 
 
 def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked, meta_stacked, indices,
-                               *, bits: int, out: torch.Tensor, accumulate: bool, blocks=None) -> torch.Tensor:
+                               *, bits: int, out: torch.Tensor, accumulate: bool, blocks=None,
+                               base_tiled=None) -> torch.Tensor:
     """T > 128: tokens are ordered by delta id on the device (dz_segment), the order is cut into
     row blocks of one delta each (dz_build_tiles) and one launch of dz_multi_delta_gemm multiplies
     every block by the base weight and by its delta in packed form.  Nothing is read back to the
     host, gathered, scattered or dequantised to memory.  `blocks`: ops.row_blocks(indices, S) when
-    the caller made it once for the batch (else made here, per call)."""
+    the caller made it once for the batch (else made here, per call).  `base_tiled`: the base weight
+    in tiles (ops.tile_base), read instead of base_weight when given."""
     from .ops import row_blocks
     T, K = x2.shape
     N = scales_stacked.shape[-1]
@@ -54,13 +56,16 @@ def multi_delta_linear_prefill(x2, base_weight, qweight_stacked, scales_stacked,
         for r in range(0, T, step):
             multi_delta_linear_prefill(x2[r:r + step], base_weight, qweight_stacked, scales_stacked, meta_stacked,
                                        indices[r:r + step].contiguous(), bits=bits, out=out[r:r + step],
-                                       accumulate=accumulate)
+                                       accumulate=accumulate, base_tiled=base_tiled)
         return out
     lib = _lib.lib()
     stream = torch.cuda.current_stream().cuda_stream
     if blocks is None:
         blocks = row_blocks(indices, S)
-    rc = lib.dz_multi_delta_gemm(x2.data_ptr(), base_weight.data_ptr() if base_weight is not None else None,
+    fn, wptr = lib.dz_multi_delta_gemm, base_weight.data_ptr() if base_weight is not None else None
+    if base_tiled is not None:
+        fn, wptr = lib.dz_multi_delta_gemm_tiled, base_tiled.data_ptr()
+    rc = fn(x2.data_ptr(), wptr,
                                  qweight_stacked.data_ptr(), meta_stacked.data_ptr(), scales_stacked.data_ptr(),
                                  S, bits, group_size, blocks.tiles.data_ptr(), blocks.max_tiles, blocks.perm.data_ptr(),
                                  out.data_ptr(), T, K, N, 1 if accumulate else 0, out.stride(0), stream)

@@ -321,6 +321,16 @@ int dz_multi_delta_gemm(const uint16_t* x, const uint16_t* w_base, const void* c
                         int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
                         uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
 
+/* dz_multi_delta_gemm with the base weight in the tiles dz_tile_base writes (the form the fused
+ * kernel reads up to 128 tokens): a layer that keeps only the tiled copy serves every batch size
+ * from it.  The same products are summed in the same order as from the row-major weight, so the
+ * results are equal bit for bit.  w_base_tiled must not be NULL (delta only: dz_multi_delta_gemm
+ * with w_base NULL).  Same reference call sites as dz_multi_delta_gemm. */
+int dz_multi_delta_gemm_tiled(const uint16_t* x, const uint16_t* w_base_tiled, const void* codes_stacked,
+                              const void* meta_stacked, const void* scales_stacked, int S, int bits,
+                              int group_size, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                              uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -110,6 +110,66 @@ def test_layer_protocol(dev):
         layer.set_delta(0, 2, p["q"][0], None, p["s"][0], None, p["m"][0])      # wrong bit width
 
 
+@pytest.mark.parametrize("t", [8, 100, 300, 700])
+def test_layer_with_only_the_tiled_base_weight(dev, t):
+    """keep_row_major_base=False: after the tiles are made the row-major weight is freed; every batch
+    size (fused kernel, its chunked form, the matrix-core kernel) reads the tiles and gives, bit for
+    bit, what a layer with both copies gives.  The parameter's loader still works."""
+    n, k, bits = 320, 1024, 2          # n is not a multiple of the matrix-core kernel's 256-feature tile
+    p = make_problem(n, k, bits, -1, 3, t, "uniform", 31 + t, dev)
+    def make(cfg):
+        lin = torch.nn.Linear(k, n, bias=False, device=dev, dtype=torch.float16)
+        with torch.no_grad():
+            lin.weight.copy_(p["wb"])
+        lin.weight.weight_loader = lambda param, loaded: param.data.copy_(loaded)
+        layer = from_layer(lin, 3, cfg, [])
+        for slot in range(3):
+            layer.set_delta(slot, bits, p["q"][slot], None, p["s"][slot], None, p["m"][slot])
+        layer.set_mapping(p["ids"], None, None, None, [t])
+        return lin, layer
+    lin_a, both = make(DeltaConfig(max_deltas=3, max_bitwidth=bits))
+    free0 = torch.cuda.memory_allocated()
+    lin_b, only = make(DeltaConfig(max_deltas=3, max_bitwidth=bits, keep_row_major_base=False))
+    assert lin_b.weight.numel() == 0 and lin_a.weight.numel() == n * k
+    assert torch.equal(only.base_tiled, both.base_tiled)
+    assert torch.equal(ops.untile_base(only.base_tiled), p["wb"])
+    ya, yb = both(p["x"])[0], only(p["x"])[0]
+    torch.cuda.synchronize()
+    assert torch.equal(ya, yb)
+    ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+    assert o.rel_err(yb.cpu().numpy(), ref) <= TOL
+    # loading another base weight through the parameter's loader: the row-major form comes back for
+    # the load and is dropped again afterwards
+    lin_b.weight.weight_loader(lin_b.weight, 2 * p["wb"])
+    assert lin_b.weight.numel() == 0
+    y2 = only(p["x"])[0]
+    torch.cuda.synchronize()
+    assert o.rel_err(y2.cpu().numpy(), o.forward_ref(p["x_np"], 2 * p["wb_np"], p["dts"], p["ids_np"])) <= TOL
+    assert torch.equal(only.restore_row_major_base(), 2 * p["wb"]) and lin_b.weight.numel() == n * k
+    with pytest.raises(ValueError):
+        DeltaConfig(tile_base_weights=False, keep_row_major_base=False)
+
+
+@pytest.mark.parametrize("bits,gs", [(2, -1), (4, 128)])
+def test_matrix_core_kernel_reads_tiles_or_rows_alike(dev, bits, gs):
+    """dz_multi_delta_gemm_tiled against dz_multi_delta_gemm on the same problem: equal bits, also
+    with fewer features than a tile and with an output slice."""
+    from deltazip_amd.prefill import multi_delta_linear_prefill
+    for n, k, t in ((96, 768, 400), (544, 1024, 1000)):
+        p = make_problem(n, k, bits, gs, 5, t, "uniform", 3 * n + bits, dev)
+        wt = ops.tile_base(p["wb"])
+        y0 = torch.zeros(t, n + 32, dtype=torch.float16, device=dev)
+        y1 = torch.zeros_like(y0)
+        multi_delta_linear_prefill(p["x"], p["wb"], p["q"], p["s"], p["m"], p["ids"], bits=bits, out=y0[:, 16:16 + n],
+                                   accumulate=False)
+        multi_delta_linear_prefill(p["x"], None, p["q"], p["s"], p["m"], p["ids"], bits=bits, out=y1[:, 16:16 + n],
+                                   accumulate=False, base_tiled=wt)
+        torch.cuda.synchronize()
+        assert torch.equal(y0, y1)
+        ref = o.forward_ref(p["x_np"], p["wb_np"], p["dts"], p["ids_np"])
+        assert o.rel_err(y1[:, 16:16 + n].cpu().numpy(), ref) <= TOL
+
+
 def test_row_parallel_rejects_bias_and_from_layer_passthrough(dev):
     lin = torch.nn.Linear(512, 64, bias=True, device=dev, dtype=torch.float16)
     cfg = DeltaConfig(max_deltas=1, max_bitwidth=4)
