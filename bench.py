@@ -238,12 +238,13 @@ def run_full_step(args, parity):
     model = LlamaForDecodeStep(mcfg, device=dev, generator=gen)
     mgr = create_delta_manager(model, max_num_seqs=T, max_num_batched_tokens=T, vocab_size=mcfg.vocab_size,
                                delta_config=DeltaConfig(max_deltas=S, max_bitwidth=bits, group_size=gs,
-                                                        tile_base_weights=not args.row_major_base))
+                                                        tile_base_weights=not args.row_major_base,
+                                                        keep_row_major_base=args.row_major_base))
     # synthetic deltas (N(0, 1e-3), compressed on the GPU) written straight into the layers' slot stacks;
     # the manager is told that delta d + 1 lives in slot d
     make_stack = random_native_stack if args.random_bits else gaussian_native_stack
     for name, layer in mgr.modules.items():
-        N, K = layer.base_layer.weight.shape
+        N, K = layer.base_shape
         layer.qweight_stacked, layer.meta_stacked, layer.scales_stacked = make_stack(K, N, bits, gs, S, dev, gen)
         layer.bitwidth = [bits] * S
     mgr.delta_index_to_id = list(range(1, S + 1))
@@ -260,15 +261,24 @@ def run_full_step(args, parity):
     # the projections alone: the same 4 x layers calls on inputs of the right shape
     projs = [m for _, m in model.projections()]
     xs = {K: torch.randn((T, K), device=dev, dtype=torch.float16, generator=gen)
-          for K in {m.base_layer.weight.shape[1] for m in projs}}
+          for K in {m.base_shape[1] for m in projs}}
 
     def linears(i):
         for m in projs:
-            m(xs[m.base_layer.weight.shape[1]])
+            m(xs[m.base_shape[1]])
     lwall, lgpu, _, _ = timed_steps(linears, steps, warmup)
     lin_ms = lgpu / steps * 1e3
-    lin_bytes = sum(algorithmic_bytes(m.base_layer.weight.shape[1], m.base_layer.weight.shape[0], T, bits, d_present)
-                    for m in projs)
+    lin_bytes = sum(algorithmic_bytes(m.base_shape[1], m.base_shape[0], T, bits, d_present) for m in projs)
+    nbytes = lambda t: t.numel() * t.element_size()
+    footprint = {
+        "base_projection_weights_bytes": sum(nbytes(m.base_layer.weight) + (nbytes(m.base_tiled) if m.base_tiled is not None
+                                                                              else 0) for m in projs),
+        "base_projection_copies": "tiles only (the row-major weight is freed once the tiles are made: "
+                                  "DeltaConfig.keep_row_major_base=False)" if not args.row_major_base else "row-major only",
+        "delta_slots_bytes": sum(nbytes(m.qweight_stacked) + nbytes(m.meta_stacked) + nbytes(m.scales_stacked) for m in projs),
+        "kv_cache_bytes": sum(nbytes(k_) + nbytes(v_) for k_, v_ in kv),
+        "allocated_bytes": torch.cuda.memory_allocated(), "reserved_bytes": torch.cuda.memory_reserved(),
+        "hbm_bytes": torch.cuda.get_device_properties(0).total_memory}
     achieved = lin_bytes / (lin_ms * 1e-3) / 1e9
     out = {
         "metric": "multi-delta linear tokens/s + achieved HBM TB/s (% peak), Llama-7B shapes",
@@ -289,6 +299,7 @@ def run_full_step(args, parity):
                      "kernel": "dz_mdl32_kernel (the projections of the step, timed on their own)",
                      "algorithmic_bytes_per_launch": lin_bytes // len(projs),
                      "avg_launch_us": round(lin_ms * 1e3 / len(projs), 2)},
+        "hbm_footprint": footprint,
         "parity": parity,
     }
     print(json.dumps(out))

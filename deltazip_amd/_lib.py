@@ -47,6 +47,7 @@ SIGNATURES = {
     "dz_gemm_f16": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16_pair": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_gemm_f16_grouped": (_i, [_vp, _vp, _vp, C.c_longlong, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp]),
+    "dz_gemm_f16_select": (_i, [_vp, _vp, _vp, C.c_longlong, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _vp]),
     "dz_set_ksplit": (None, [_i]),
     "dz_probe_read": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp]),
 }

@@ -34,8 +34,10 @@ struct GemmParams {
   const _Float16* w2;            // stack of second weights or nullptr
   long long w2_stride;           // elements between consecutive second weights
   const dz_gemm_tile* tiles;     // row blocks, or nullptr: blocks of 256 rows, second weight 0
+  const int* perm;               // row blocks count positions of this token order (rows of x and y), or nullptr
   _Float16* y;
   int T, K, N, accumulate, ldy, tiles_m, tiles_n;
+  int select;                    // a block with a second weight is multiplied by that weight only
 };
 
 __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
@@ -60,9 +62,15 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
   const int n0 = tn * BN;
   const _Float16* w2 = (P.w2 && widx >= 0) ? P.w2 + (size_t)widx * P.w2_stride : nullptr;
   const int nslab1 = P.K / BK, nslab = w2 ? 2 * nslab1 : nslab1;
-  const int s_begin = P.w ? 0 : nslab1;   // no first weight: second product only
+  const int s_begin = (P.w && !(P.select && w2)) ? 0 : nslab1;   // no first weight (for this block): second product only
   if (s_begin >= nslab) return;           // neither: the tile is left as it is
   const unsigned Kb = (unsigned)P.K * 2u;
+  // A block of few rows (a decode batch spread over several tables): token rows beyond the block
+  // are neither requested nor multiplied -- a request covers 8 rows, a product 32 -- so that such a
+  // block costs the stream of its weight slab and little else.  (What the skipped rows' LDS bytes
+  // hold only reaches output columns that are never stored.)
+  const int nrows = row_hi - row_lo;
+  const int nb = min(4, max(0, (nrows - wm * 128 + 31) / 32));   // this wavefront's 32-token tiles in use
 
   f16_t acc[4][4];
 #pragma unroll
@@ -83,7 +91,10 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
     const int rq = wave * 16 + i, sub = rq & 31, R = sub * 8 + lr;
     unsigned rowoff;
     if (rq < 32) rowoff = (unsigned)min(n0 + R, P.N - 1);           // weight rows (clamped: never stored)
-    else rowoff = (unsigned)min(row_lo + R, row_hi - 1);            // token rows
+    else {                                                          // token rows
+      const int pos = min(row_lo + R, row_hi - 1);
+      rowoff = (unsigned)(P.perm ? P.perm[pos] : pos);
+    }
     const int lc = (lane & 7) ^ ((R >> 1) & 7);
     goff[i] = rowoff * Kb + (unsigned)lc * 16u;
   }
@@ -103,7 +114,9 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
       const int rq = wave * 16 + i, sub = rq & 31;
       unsigned char* dst = smem + buf * (2 * SLAB) + (rq < 32 ? 0 : SLAB) + sub * 1024;
       __attribute__((address_space(3))) void* d3 = (__attribute__((address_space(3))) void*)dst;
-      if (rq >= 32) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, d3, 16, (int)goff[i], soff, 0, 0);
+      if (rq >= 32) {
+        if (sub * 8 < nrows) __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, d3, 16, (int)goff[i], soff, 0, 0);
+      }
       else if (second) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw2, d3, 16, (int)goff[i], soff, 0, 0);
       else __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, d3, 16, (int)goff[i], soff, 0, 0);
     }
@@ -133,21 +146,25 @@ __global__ __launch_bounds__(256, 1) void dz_gemm_kernel(const GemmParams P) {
 #pragma unroll
       for (int a = 0; a < 4; ++a) fw[a] = *(const h8_t*)(wb + wrow + a * 32 * 128 + foff[kk]);
 #pragma unroll
-      for (int b = 0; b < 4; ++b) fx[b] = *(const h8_t*)(xb + xrow + b * 32 * 128 + foff[kk]);
+      for (int b = 0; b < 4; ++b)
+        if (b < nb) fx[b] = *(const h8_t*)(xb + xrow + b * 32 * 128 + foff[kk]);
       // operand order (w, x): result rows = output features, columns = tokens, so each lane ends
       // up with 4 consecutive output features of one token = one 8-byte store
 #pragma unroll
-      for (int a = 0; a < 4; ++a)
+      for (int b = 0; b < 4; ++b)
+        if (b < nb) {
 #pragma unroll
-        for (int b = 0; b < 4; ++b)
-          acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[a], fx[b], acc[a][b], 0, 0, 0);
+          for (int a = 0; a < 4; ++a)
+            acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[a], fx[b], acc[a][b], 0, 0, 0);
+        }
     }
   }
 
 #pragma unroll
   for (int b = 0; b < 4; ++b) {
-    const int tok = row_lo + wm * 128 + b * 32 + li;
-    if (tok >= row_hi) continue;
+    const int pos = row_lo + wm * 128 + b * 32 + li;
+    if (pos >= row_hi) continue;
+    const int tok = P.perm ? P.perm[pos] : pos;
 #pragma unroll
     for (int a = 0; a < 4; ++a) {
       // The accumulators live in the accumulation registers; pinning each block there until its
@@ -228,5 +245,14 @@ extern "C" int dz_gemm_f16_grouped(const uint16_t* x, const uint16_t* w, const u
   if (!tiles || ntiles < 1) return DZ_EINVAL;
   GemmParams P = base_params(x, w, y, T, K, N, accumulate, ldy);
   P.w2 = (const _Float16*)w2_stack; P.w2_stride = w2_stride; P.tiles = tiles;
+  return gemm_launch(P, ntiles, stream);
+}
+
+extern "C" int dz_gemm_f16_select(const uint16_t* x, const uint16_t* w_base, const uint16_t* w_stack,
+                                  long long w_stride, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                                  uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream) {
+  if (!tiles || ntiles < 1 || !w_base || !w_stack) return DZ_EINVAL;
+  GemmParams P = base_params(x, w_base, y, T, K, N, accumulate, ldy);
+  P.w2 = (const _Float16*)w_stack; P.w2_stride = w_stride; P.tiles = tiles; P.perm = perm; P.select = 1;
   return gemm_launch(P, ntiles, stream);
 }

@@ -78,6 +78,7 @@ class LinearWithDelta(BaseLayerWithDelta):
         if w.dtype != torch.float16 or w.dim() != 2:
             raise ValueError("base layer weight must be float16 [out_features, in_features]")
         N, K = w.shape
+        self.base_shape = (N, K)      # stays when the row-major weight is freed (keep_row_major_base=False)
         self.bits = delta_config.max_bitwidth
         self.pack_factor = delta_config.pack_factor
         self.group_size = delta_config.group_size

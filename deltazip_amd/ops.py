@@ -214,9 +214,10 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     (serving/vllm/delta/deltazip_marlin.py:21-53, the lm_head of LogitsProcessorWithDelta):
     out[t] = x[t] @ delta_weights[indices[t]]^T, or x[t] @ base_embedding^T for indices[t] == -1.
     Where the reference loops over torch.unique(indices) on the host, the rows are grouped by id
-    and cut into row blocks on the device (dz_segment, dz_build_tiles) and two grouped launches
-    multiply them -- the blocks without a delta by the base table, the others by their delta's --
-    so nothing is read back to the host and the call can be captured in a HIP graph."""
+    and cut into row blocks on the device (dz_segment, dz_build_tiles) and one launch multiplies
+    every block by its own table (dz_gemm_f16_select), reading and writing the rows in place
+    through the token order: three launches, nothing gathered, scattered or read back to the
+    host, so the call can be captured in a HIP graph."""
     _need_cuda(x, delta_weights, indices, base_embedding)
     if x.dtype != torch.float16 or delta_weights.dtype != torch.float16 or base_embedding.dtype != torch.float16:
         raise ValueError("x and the weights must be float16")
@@ -224,28 +225,13 @@ def apply_delta_uncompressed(x: torch.Tensor, delta_weights: torch.Tensor, indic
     T = x.shape[0]
     if x.dim() != 2 or x.shape[1] != K or tuple(base_embedding.shape) != (N, K) or indices.numel() != T:
         raise ValueError("shapes: x [T, K], delta_weights [S, N, K], base_embedding [N, K], indices [T]")
-    if not (delta_weights.is_contiguous() and base_embedding.is_contiguous()):
-        raise ValueError("weights must be contiguous")
-    lib, st = _lib.lib(), _stream()
-    perm, seg_off = segment(indices.contiguous(), S)
-    max_tiles = (T + 255) // 256 + min(S + 1, T)
-    tiles = torch.empty((max_tiles, 4), dtype=torch.int32, device=x.device)
-    _lib.check(lib.dz_build_tiles(seg_off.data_ptr(), S, tiles.data_ptr(), max_tiles, st), "dz_build_tiles")
-    # two copies of the block table: one keeps the blocks without a delta, one the others (a block
-    # whose row range is empty is skipped by the kernel)
-    with_delta = tiles[:, 2] >= 0
-    base_tiles, delta_tiles = tiles.clone(), tiles.clone()
-    base_tiles[:, 1] = torch.where(with_delta, tiles[:, 0], tiles[:, 1])
-    delta_tiles[:, 1] = torch.where(with_delta, tiles[:, 1], tiles[:, 0])
-    perm64 = perm.long()
-    xs = x.index_select(0, perm64)
-    ys = torch.empty((T, N), dtype=torch.float16, device=x.device)
-    _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), base_embedding.data_ptr(), None, N * K, base_tiles.data_ptr(),
-                                       max_tiles, ys.data_ptr(), T, K, N, 0, N, st), "dz_gemm_f16_grouped")
-    _lib.check(lib.dz_gemm_f16_grouped(xs.data_ptr(), None, delta_weights.data_ptr(), N * K, delta_tiles.data_ptr(),
-                                       max_tiles, ys.data_ptr(), T, K, N, 0, N, st), "dz_gemm_f16_grouped")
-    out = torch.empty_like(ys)
-    out.index_copy_(0, perm64, ys)
+    if not (delta_weights.is_contiguous() and base_embedding.is_contiguous() and x.is_contiguous()):
+        raise ValueError("x and the weights must be contiguous")
+    blocks = row_blocks(indices, S)
+    out = torch.empty((T, N), dtype=torch.float16, device=x.device)
+    _lib.check(_lib.lib().dz_gemm_f16_select(x.data_ptr(), base_embedding.data_ptr(), delta_weights.data_ptr(), N * K,
+                                             blocks.tiles.data_ptr(), blocks.max_tiles, blocks.perm.data_ptr(),
+                                             out.data_ptr(), T, K, N, 0, N, _stream()), "dz_gemm_f16_select")
     return out
 
 

@@ -299,6 +299,19 @@ int dz_gemm_f16_grouped(const uint16_t* x, const uint16_t* w, const uint16_t* w2
                         long long w2_stride, const dz_gemm_tile* tiles, int ntiles, uint16_t* y,
                         int T, int K, int N, int accumulate, int ldy, void* stream);
 
+/* Per-row choice of one full weight: for every row block b of `tiles` and every position p in
+ * [row_lo, row_hi), with t = perm ? perm[p] : p,
+ *   y[t, 0..N) (+)= x[t] @ (group(b) >= 0 ? w_stack[group(b)] : w_base)^T
+ * -- the output projection of the reference's LogitsProcessorWithDelta, whose
+ * apply_delta_uncompressed loops over torch.unique(indices) on the host and multiplies each id's
+ * rows by that delta's own table, the rows without a delta by the base table
+ * (serving/vllm/delta/deltazip_marlin.py:21-53).  With perm = what dz_segment wrote and tiles =
+ * what dz_build_tiles wrote, the whole call is three launches and nothing is gathered, scattered
+ * or read back.  Rows outside every block are not written. */
+int dz_gemm_f16_select(const uint16_t* x, const uint16_t* w_base, const uint16_t* w_stack,
+                       long long w_stride, const dz_gemm_tile* tiles, int ntiles, const int32_t* perm,
+                       uint16_t* y, int T, int K, int N, int accumulate, int ldy, void* stream);
+
 /* Row blocks for dz_multi_delta_gemm from the segment offsets dz_segment wrote (device memory,
  * S + 2 entries): every segment is cut into blocks of at most 256 rows, group = slot (-1 for the
  * tokens without a delta); entries of `tiles` (device memory, max_tiles of them) beyond the blocks
