@@ -1,11 +1,14 @@
 """Slot manager: which delta sits in which GPU slot, and the per-batch index tensors.
 
-Mirrors serving/vllm/delta/models.py of eth-easl/deltazip:
+Stands in for serving/vllm/delta/models.py of eth-easl/deltazip, with its public names:
   :69-145    convert_mapping          (here: one H2D copy of the raw ids + one kernel, dz_map_ids,
                                        instead of a Python loop doing list.index per token)
   :266-503   DeltaModelManager        activate / deactivate / add / remove / set_delta_mapping,
                                        module replacement through `from_layer`
-  :533-603   DeltaLRUCache, LRUCacheDeltaModelManager, create_delta_manager
+  :533-603   LRUCacheDeltaModelManager, create_delta_manager
+The bookkeeping is one class with two tiers (host, slots) of the same small container and an
+eviction policy flag, rather than a base manager plus a subclass that swaps its dictionaries for
+caches with removal callbacks.
 
 The manager owns the index buffers; the layers hold views of them (`set_mapping`), and the kernels
 read them on the device when a layer runs.  `activate_delta` copies a delta's native-layout
@@ -16,11 +19,7 @@ it has one).
 """
 from __future__ import annotations
 
-import copy
-import math
-import re
-from collections import OrderedDict
-from typing import Any, Callable, Dict, Hashable, List, Optional, Type
+from typing import Any, Dict, Hashable, List, Optional, Type
 
 import torch
 import torch.nn as nn
@@ -32,17 +31,21 @@ from .layers import BaseLayerWithDelta, DeltaMapping, LinearWithDelta, from_laye
 
 
 class LRUCache:
-    """serving/vllm/utils.py:62-130."""
+    """Bounded mapping that forgets its least recently used entry; same interface as the helper the
+    serving engine uses (serving/vllm/utils.py:62-130: `get` / `put` / `touch` / `pop` /
+    `remove_oldest` / `clear`, `_on_remove(key, value)` as the hook for subclasses).  Built on the
+    insertion order of a plain dict: the first key is the oldest, using a key re-inserts it."""
 
     def __init__(self, capacity: int):
-        self.cache: "OrderedDict[Hashable, Any]" = OrderedDict()
         self.capacity = capacity
+        self._entries: Dict[Hashable, Any] = {}
 
+    # container protocol
     def __contains__(self, key: Hashable) -> bool:
-        return key in self.cache
+        return key in self._entries
 
     def __len__(self) -> int:
-        return len(self.cache)
+        return len(self._entries)
 
     def __getitem__(self, key: Hashable):
         return self.get(key)
@@ -54,66 +57,124 @@ class LRUCache:
         self.pop(key)
 
     def keys(self):
-        return self.cache.keys()
+        return self._entries.keys()
 
+    @property
+    def cache(self) -> Dict[Hashable, Any]:
+        return self._entries
+
+    # recency
     def touch(self, key: Hashable) -> None:
-        self.cache.move_to_end(key)
+        self._entries[key] = self._entries.pop(key)
 
     def get(self, key: Hashable, default_value=None):
-        if key in self.cache:
-            self.cache.move_to_end(key)
-            return self.cache[key]
-        return default_value
+        if key not in self._entries:
+            return default_value
+        self.touch(key)
+        return self._entries[key]
 
     def put(self, key: Hashable, value) -> None:
-        self.cache[key] = value
-        self.cache.move_to_end(key)
-        while len(self.cache) > self.capacity:
+        self._entries.pop(key, None)
+        self._entries[key] = value
+        while len(self._entries) > self.capacity:
             self.remove_oldest()
 
+    # removal: every entry that leaves passes through the hook exactly once
     def _on_remove(self, key: Hashable, value) -> None:
         pass
 
     def remove_oldest(self) -> None:
-        if not self.cache:
+        for key in self._entries:
+            self._on_remove(key, self._entries.pop(key))
             return
-        key, value = self.cache.popitem(last=False)
-        self._on_remove(key, value)
 
     def pop(self, key: Hashable, default_value=None):
-        run_on_remove = key in self.cache
-        value = self.cache.pop(key, default_value)
-        if run_on_remove:
-            self._on_remove(key, value)
+        if key not in self._entries:
+            return default_value
+        value = self._entries.pop(key)
+        self._on_remove(key, value)
         return value
 
     def clear(self) -> None:
-        while len(self.cache) > 0:
+        while self._entries:
             self.remove_oldest()
-        self.cache.clear()
 
 
 def replace_submodule(model: nn.Module, module_name: str, new_module: nn.Module) -> nn.Module:
-    """serving/vllm/delta/utils.py: swap a sub-module by dotted name."""
-    parent = model.get_submodule(".".join(module_name.split(".")[:-1]))
-    setattr(parent, module_name.split(".")[-1], new_module)
+    """Puts `new_module` where the dotted name points (serving/vllm/delta/utils.py)."""
+    parent_name, _, leaf = module_name.rpartition(".")
+    setattr(model.get_submodule(parent_name), leaf, new_module)
     return new_module
 
 
+class _Recency:
+    """id -> value, remembered in order of last use (oldest first).  The manager's two sets -- the
+    deltas registered in host memory and the deltas resident in GPU slots -- are one of these each;
+    whether the oldest entry may be pushed out to make room is the manager's policy, not the
+    container's."""
+
+    def __init__(self) -> None:
+        self._d: Dict[int, Any] = {}
+
+    def __contains__(self, key: int) -> bool:
+        return key in self._d
+
+    def __len__(self) -> int:
+        return len(self._d)
+
+    def __iter__(self):
+        return iter(self._d)
+
+    def peek(self, key: int, default=None):
+        return self._d.get(key, default)
+
+    def use(self, key: int):
+        value = self._d[key] = self._d.pop(key)
+        return value
+
+    def add(self, key: int, value) -> None:
+        self._d.pop(key, None)
+        self._d[key] = value
+
+    def drop(self, key: int, default=None):
+        return self._d.pop(key, default)
+
+    def oldest(self) -> Optional[int]:
+        return next(iter(self._d), None)
+
+    def snapshot(self) -> Dict[int, Any]:
+        return dict(self._d)
+
+    def clear(self) -> None:
+        self._d.clear()
+
+
 class DeltaModelManager:
-    """A manager that manages multiple full-fine-tuned models (delta/models.py:266-503)."""
+    """Keeps fine-tuned deltas in two tiers -- registered in (pinned) host memory, resident in one of
+    the GPU slots of every wrapped layer -- and turns a batch's delta ids into the index tensors the
+    layers read (the role of serving/vllm/delta/models.py:266-503; same public methods).
+
+    `evict_lru = False`: a full tier refuses (`add_delta` raises RuntimeError, `activate_delta`
+    raises ValueError), as the reference's plain manager does.  `evict_lru = True`
+    (`LRUCacheDeltaModelManager`): the least recently used entry of the full tier makes room; a
+    delta that leaves the host tier also leaves its slot."""
+
+    evict_lru = False
 
     def __init__(self, model: nn.Module, max_num_seqs: int, max_num_batched_tokens: int, vocab_size: int,
                  delta_config: DeltaConfig, device: Optional[torch.device] = None) -> None:
         self.delta_config = delta_config
         self.max_num_seqs = max_num_seqs
-        assert self.capacity >= self.delta_slots, "capacity must be greater than delta_slots"
-        self.max_num_batched_tokens = math.ceil(max_num_batched_tokens / 8) * 8
-        self.delta_index_to_id: List[Optional[int]] = [None] * self.delta_slots
+        if self.capacity < self.delta_slots:
+            raise AssertionError("capacity must be greater than delta_slots")
+        self.max_num_batched_tokens = -(-max_num_batched_tokens // 8) * 8
         self.vocab_size = vocab_size
-        if device is None:
-            device = next(model.parameters()).device
-        self.device = torch.device(device)
+        self.device = torch.device(device if device is not None else next(model.parameters()).device)
+        # the two tiers; `_slot_ids[i]` = id of the delta resident in slot i (public name:
+        # delta_index_to_id, as in the reference)
+        self._host = _Recency()          # id -> DeltaModel
+        self._resident = _Recency()      # id -> slot
+        self._slot_ids: List[Optional[int]] = [None] * self.delta_slots
         n = self.max_num_batched_tokens
         self.base_indices = torch.empty(n, dtype=torch.long, device=self.device)
         self.sampler_indices = torch.empty(n, dtype=torch.long, device=self.device)
@@ -136,23 +197,19 @@ class DeltaModelManager:
         self._staged = torch.cuda.Event() if pin else None    # last copy out of the pinned buffers
         self.indices_len: List[int] = []
         self.model = model
-        self.supported_delta_modules: List[str] = []
-        self.packed_modules_mapping: Dict[str, List[str]] = {}
-        if hasattr(self.model, "supported_delta_modules"):
-            self.supported_delta_modules = copy.deepcopy(self.model.supported_delta_modules)
-            self.packed_modules_mapping = copy.deepcopy(getattr(self.model, "packed_modules_mapping", {}))
-        # llama.py:336-339 of the serving model
-        self.embedding_modules = dict(getattr(self.model, "embedding_modules",
+        # which sub-modules carry deltas: the model says so (llama.py:336-339 of the serving model)
+        self.supported_delta_modules: List[str] = list(getattr(model, "supported_delta_modules", []))
+        self.packed_modules_mapping: Dict[str, List[str]] = {
+            k: list(v) for k, v in getattr(model, "packed_modules_mapping", {}).items()}
+        self.embedding_modules = dict(getattr(model, "embedding_modules",
                                               {"embed_tokens": "input_embeddings", "lm_head": "output_embeddings"}))
         self.packed_modules: Dict[str, List[str]] = {}
         self.modules: Dict[str, BaseLayerWithDelta] = {}
-        self._registered_deltas: Dict[int, DeltaModel] = {}
-        self._active_deltas: Dict[int, None] = {}
         self._last_mapping: Optional[DeltaMapping] = None
-        self._create_delta_modules()
+        self._wrap_modules()
         self.model.delta_manager = self
 
-    # -- bookkeeping -----------------------------------------------------------------------
+    # -- the two tiers -----------------------------------------------------------------------
     @property
     def capacity(self) -> int:
         return self.delta_config.max_cpu_deltas
@@ -161,78 +218,112 @@ class DeltaModelManager:
     def delta_slots(self) -> int:
         return self.delta_config.max_deltas
 
-    def __len__(self) -> int:
-        return len(self._registered_deltas)
+    @property
+    def delta_index_to_id(self) -> List[Optional[int]]:
+        return self._slot_ids
 
-    def activate_delta(self, delta_id: int) -> bool:
-        """Move a delta into the GPU slots to be used in the forward pass."""
-        if delta_id in self._active_deltas:
-            return False
-        index = next((i for i, d in enumerate(self.delta_index_to_id) if d is None), None)
-        if index is None:
-            raise ValueError("No free delta slots")
-        self._active_deltas[delta_id] = None
-        delta_model = self._registered_deltas[delta_id]
-        self.delta_index_to_id[index] = delta_model.id
+    @delta_index_to_id.setter
+    def delta_index_to_id(self, ids) -> None:
+        # for callers that fill the layers' slot stacks themselves (synthetic benchmarks)
+        ids = list(ids)
+        if len(ids) != self.delta_slots:
+            raise ValueError("one entry per slot")
+        self._slot_ids[:] = ids
+        self._resident.clear()
+        for slot, d in enumerate(ids):
+            if d is not None:
+                self._resident.add(d, slot)
+        self._slots_changed()
+
+    def __len__(self) -> int:
+        return len(self._host)
+
+    def _slots_changed(self) -> None:
         self._slots_dirty = True
         self._last_mapping = None     # slot numbers may have changed under an unchanged mapping
-        for module_name, module in self.modules.items():
-            module_delta = delta_model.get_delta(module_name)
-            if module_delta is None:
-                module.reset_delta(index)
-            elif module_delta._compressed:
-                module.set_delta(index, delta_model.bitwidth, module_delta.qweight, module_delta.qzeros,
-                                 module_delta.scales, module_delta.g_idx, module_delta.meta)
+
+    def _vacate(self, delta_id: int) -> Optional[int]:
+        """Takes a delta out of the resident tier; returns the slot it held.  The slot's tensors stay
+        as they are: nothing points at them until the next delta is written there."""
+        slot = self._resident.drop(delta_id)
+        if slot is not None:
+            self._slot_ids[slot] = None
+            self._slots_changed()
+        return slot
+
+    def _write_slot(self, slot: int, delta_model: DeltaModel) -> None:
+        for name, module in self.modules.items():
+            part = delta_model.get_delta(name)
+            if part is None:
+                module.reset_delta(slot)
+            elif part._compressed:
+                module.set_delta(slot, delta_model.bitwidth, part.qweight, part.qzeros, part.scales, part.g_idx,
+                                 part.meta)
             else:
-                module.set_delta(index, delta_model.bitwidth, module_delta.weight)
+                module.set_delta(slot, delta_model.bitwidth, part.weight)
+
+    def activate_delta(self, delta_id: int) -> bool:
+        """Makes a registered delta resident: picks a slot (the lowest free one; with `evict_lru` the
+        least recently activated delta's when none is free) and copies the delta's tensors into that
+        slot of every wrapped layer.  False if it was resident already."""
+        if delta_id in self._resident:
+            self._resident.use(delta_id)
+            return False
+        if None not in self._slot_ids and not self.evict_lru:
+            raise ValueError("No free delta slots")
+        delta_model = self._host.use(delta_id)       # KeyError for an id that was never added
+        if None not in self._slot_ids:
+            self._vacate(self._resident.oldest())
+        slot = self._slot_ids.index(None)
+        self._slot_ids[slot] = delta_model.id
+        self._resident.add(delta_id, slot)
+        self._slots_changed()
+        self._write_slot(slot, delta_model)
         return True
 
     def _deactivate_delta(self, delta_id: int) -> None:
-        try:
-            index = self.delta_index_to_id.index(delta_id)
-            self.delta_index_to_id[index] = None
-            self._slots_dirty = True
-            self._last_mapping = None
-        except ValueError:
-            pass
+        self._vacate(delta_id)
 
     def deactivate_delta(self, delta_id: int) -> bool:
-        """Remove a delta from its GPU slot."""
-        if delta_id in self._active_deltas:
-            self._deactivate_delta(delta_id)
-            self._active_deltas.pop(delta_id)
-            return True
-        return False
-
-    def _add_delta(self, delta: DeltaModel) -> None:
-        self._registered_deltas[delta.id] = delta
+        """Takes a delta out of its GPU slot; False if it had none."""
+        return self._vacate(delta_id) is not None
 
     def add_delta(self, delta: DeltaModel) -> bool:
-        """Add a DeltaModel to the manager's host cache."""
-        if delta.id not in self._registered_deltas:
-            if len(self._registered_deltas) >= self.capacity:
+        """Registers a DeltaModel in the host tier; False if its id is registered already."""
+        if delta.id in self._host:
+            if self.evict_lru:
+                self._host.use(delta.id)
+            return False
+        if len(self._host) >= self.capacity:
+            if not self.evict_lru:
                 raise RuntimeError("No free Delta slots.")
-            self._add_delta(delta)
-            return True
-        return False
+            self.remove_oldest_delta()
+        self._host.add(delta.id, delta)
+        return True
 
     def remove_delta(self, delta_id: int) -> bool:
-        """Remove a DeltaModel from the manager's host cache."""
-        self.deactivate_delta(delta_id)
-        return bool(self._registered_deltas.pop(delta_id, None))
+        """Forgets a delta: out of its slot, out of the host tier."""
+        self._vacate(delta_id)
+        return self._host.drop(delta_id) is not None
+
+    def remove_oldest_delta(self) -> bool:
+        """Forgets the registered delta that was used longest ago."""
+        oldest = self._host.oldest()
+        return oldest is not None and self.remove_delta(oldest)
 
     def list_deltas(self) -> Dict[int, DeltaModel]:
-        return dict(self._registered_deltas)
+        return self._host.snapshot()
 
     def get_delta(self, delta_id: int) -> Optional[DeltaModel]:
-        return self._registered_deltas.get(delta_id, None)
+        if delta_id not in self._host:
+            return None
+        return self._host.use(delta_id) if self.evict_lru else self._host.peek(delta_id)
 
     def remove_all_deltas(self) -> None:
-        self._registered_deltas.clear()
-        self.delta_index_to_id = [None] * self.delta_slots
-        self._active_deltas.clear()
-        self._slots_dirty = True
-        self._last_mapping = None
+        self._host.clear()
+        self._resident.clear()
+        self._slot_ids[:] = [None] * self.delta_slots
+        self._slots_changed()
 
     # -- the per-batch mapping -------------------------------------------------------------
     def _set_delta_mapping(self, mapping: DeltaMapping) -> None:
@@ -293,105 +384,62 @@ class DeltaModelManager:
         self._last_mapping = delta_mapping
 
     # -- module replacement ----------------------------------------------------------------
-    def _create_delta_modules(self) -> None:
-        for module_name, module in list(self.model.named_modules()):
-            if not self._match_target_modules(module_name):
+    def _is_target(self, module_name: str) -> bool:
+        """A module carries deltas when its dotted name is, or ends in, one of the model's
+        `supported_delta_modules`."""
+        return any(module_name == t or module_name.endswith("." + t) for t in self.supported_delta_modules)
+
+    def _wrap_modules(self) -> None:
+        """Swaps every target sub-module for its delta-carrying counterpart and hands it the index
+        buffers.  The output projection is special: its per-delta tables live in the model's
+        `logits_processor` (delta/models.py:467-479), which is wrapped in its stead and registered
+        under the projection's name."""
+        model_config = getattr(self.model, "config", None)
+        for name, module in list(self.model.named_modules()):
+            if not self._is_target(name):
                 continue
-            last = module_name.split(".")[-1]
-            model_config = getattr(self.model, "config", None)
-            if self.embedding_modules.get(last) == "output_embeddings":
-                # the output projection's delta lives in the logits processor (models.py:467-479)
-                try:
-                    logits_processor = self.model.get_submodule("logits_processor")
-                except AttributeError:
+            leaf = name.rpartition(".")[2]
+            if self.embedding_modules.get(leaf) == "output_embeddings":
+                if not hasattr(self.model, "logits_processor"):
                     continue
-                new_module = replace_submodule(
-                    self.model, "logits_processor",
-                    from_layer_logits_processor(logits_processor, module, self.delta_slots, self.delta_config,
-                                                model_config))
+                wrapped = from_layer_logits_processor(self.model.logits_processor, module, self.delta_slots,
+                                                      self.delta_config, model_config)
+                replace_submodule(self.model, "logits_processor", wrapped)
             else:
-                packed = self.packed_modules_mapping.get(last, [])
-                new_module = from_layer(module, self.delta_slots, self.delta_config, packed, model_config)
-                if not isinstance(new_module, BaseLayerWithDelta):
-                    continue
-                replace_submodule(self.model, module_name, new_module)
-            self.register_module(module_name, new_module)
-            self._register_packed_modules(module_name)
-            if isinstance(new_module, LinearWithDelta):
-                new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
-                                       self.embeddings_indices, self.indices_len, token_order=self.token_order,
-                                       row_blocks=self.row_blocks)
-            else:
-                new_module.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
-                                       self.embeddings_indices, self.indices_len)
+                wrapped = from_layer(module, self.delta_slots, self.delta_config,
+                                     self.packed_modules_mapping.get(leaf, []), model_config)
+                if not isinstance(wrapped, BaseLayerWithDelta):
+                    continue        # from_layer hands back what it cannot wrap
+                replace_submodule(self.model, name, wrapped)
+            self.register_module(name, wrapped)
+            extra = ({"token_order": self.token_order, "row_blocks": self.row_blocks}
+                     if isinstance(wrapped, LinearWithDelta) else {})
+            wrapped.set_mapping(self.base_indices, self.sampler_indices, self.sampler_indices_padded,
+                                self.embeddings_indices, self.indices_len, **extra)
 
     def register_module(self, module_name: str, module: BaseLayerWithDelta) -> None:
-        assert isinstance(module, BaseLayerWithDelta)
+        if not isinstance(module, BaseLayerWithDelta):
+            raise TypeError("only delta-carrying layers are registered")
         self.modules[module_name] = module
-
-    def _match_target_modules(self, module_name: str) -> bool:
-        return any(re.match(r".*\.{target_module}$".format(target_module=t), module_name) or t == module_name
-                   for t in self.supported_delta_modules)
-
-    def _register_packed_modules(self, module_full_name: str) -> None:
-        parts = module_full_name.split(".")
-        replacements = self.packed_modules_mapping.get(parts[-1])
-        if not replacements:
-            return
-        prefix = ".".join(parts[:-1])
-        self.packed_modules[module_full_name] = [prefix + "." + r if prefix else r for r in replacements]
-
-
-class DeltaLRUCache(LRUCache):
-    def __init__(self, capacity: int, deactivate_delta_fn: Callable[[Hashable], None]):
-        super().__init__(capacity)
-        self.deactivate_delta_fn = deactivate_delta_fn
-
-    def _on_remove(self, key: Hashable, value) -> None:
-        self.deactivate_delta_fn(key)
-        return super()._on_remove(key, value)
+        # a fused layer also answers for the projections it is made of (q/k/v, gate/up)
+        parent, _, leaf = module_name.rpartition(".")
+        parts = self.packed_modules_mapping.get(leaf)
+        if parts:
+            self.packed_modules[module_name] = [f"{parent}.{part}" if parent else part for part in parts]
 
 
 class LRUCacheDeltaModelManager(DeltaModelManager):
-    """A manager that evicts the least recently used delta (delta/models.py:546-603)."""
+    """The manager with both tiers evicting their least recently used delta
+    (role of delta/models.py:546-603)."""
 
-    def __init__(self, model: nn.Module, max_num_seqs: int, max_num_batched_tokens: int, vocab_size: int,
-                 delta_config: DeltaConfig, device: Optional[torch.device] = None):
-        super().__init__(model, max_num_seqs, max_num_batched_tokens, vocab_size, delta_config, device)
-        self._registered_deltas = DeltaLRUCache(self.capacity, self.deactivate_delta)
-        self._active_deltas = DeltaLRUCache(self.delta_slots, self._deactivate_delta)
-
-    def list_deltas(self) -> Dict[int, DeltaModel]:
-        return dict(self._registered_deltas.cache)
-
-    def add_delta(self, delta: DeltaModel) -> bool:
-        if delta.id not in self._registered_deltas:
-            self._add_delta(delta)
-            return True
-        self._registered_deltas.touch(delta.id)   # always touch to update the LRU order
-        return False
-
-    def activate_delta(self, delta_id: int) -> bool:
-        if delta_id not in self._active_deltas and len(self._active_deltas) >= self.delta_slots:
-            self._active_deltas.remove_oldest()
-        result = super().activate_delta(delta_id)
-        self._active_deltas.touch(delta_id)
-        return result
-
-    def remove_oldest_delta(self) -> bool:
-        if len(self._registered_deltas) > 0:
-            self._registered_deltas.remove_oldest()
-            return True
-        return False
+    evict_lru = True
 
 
 def create_delta_manager(model: nn.Module, max_num_seqs: int, max_num_batched_tokens: int, vocab_size: int,
                          delta_config: DeltaConfig,
                          delta_manager_cls: Type[DeltaModelManager] = DeltaModelManager,
                          **kwargs) -> DeltaModelManager:
-    """Create a delta manager for a given model (delta/models.py:606-626)."""
+    """Wraps the model's delta modules and returns their manager (delta/models.py:606-626)."""
     if not hasattr(model, "supported_delta_modules"):
         raise ValueError(f"Model {type(model)} is not supported for Delta.")
-    return delta_manager_cls(model=model, max_num_seqs=max_num_seqs,
-                             max_num_batched_tokens=max_num_batched_tokens, vocab_size=vocab_size,
-                             delta_config=delta_config, **kwargs)
+    return delta_manager_cls(model, max_num_seqs, max_num_batched_tokens, vocab_size, delta_config, **kwargs)
