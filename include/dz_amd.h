@@ -213,7 +213,10 @@ int dz_multi_delta_linear(const uint16_t* x, const uint16_t* w_base,
  * call on a device looks the array's address up (hipGetSymbolAddress), which is the only set-up.
  * All calls on one GPU share the array: calls that overlap in time on one GPU (two streams, two
  * host threads) race; order them on one stream.  The array is all zero bits at load and every
- * call leaves the partial-sum slots zero again, as with a caller's workspace. */
+ * call leaves the partial-sum slots zero again, as with a caller's workspace.  The status word
+ * inside the array cannot be read back through this interface: a caller that wants to see a bad
+ * token id or a failed exchange of partial sums reported (and the slots emptied after one) uses
+ * dz_multi_delta_linear with a workspace of its own. */
 int dz_multi_delta_linear_static(const uint16_t* x, const uint16_t* w_base,
                                  const void* codes_stacked, const void* meta_stacked,
                                  const void* scales_stacked, const int64_t* indices, uint16_t* y,
