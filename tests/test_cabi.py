@@ -68,6 +68,26 @@ def test_argument_checks_happen_on_the_host(dzlib):
     assert mp(one, 4, None, 0, one, 2, 3, 100, 0, one, None, None, one, 3, None, None) == -2
     assert dzlib.dz_gemm_f16(one, one, one, 8, 100, 128, 0, 128, None) == -2
     assert dzlib.dz_gemm_f16(None, one, one, 8, 128, 128, 0, 128, None) == -1
+    # the per-row table choice and the tiled form of the prefill entry point: missing tables / tiles
+    sel = dzlib.dz_gemm_f16_select
+    assert sel(one, one, one, 64 * 256, None, 4, one, one, 8, 256, 64, 0, 64, None) == -1      # no row blocks
+    assert sel(one, None, one, 64 * 256, one, 4, one, one, 8, 256, 64, 0, 64, None) == -1     # no base table
+    assert sel(one, one, None, 64 * 256, one, 4, one, one, 8, 256, 64, 0, 64, None) == -1     # no delta tables
+    gt = dzlib.dz_multi_delta_gemm_tiled
+    assert gt(one, None, one, one, one, 2, 4, -1, one, 4, None, one, 300, 512, 64, 0, 64, None) == -1
+    assert gt(one, one, one, one, one, 2, 3, -1, one, 4, None, one, 300, 512, 64, 0, 64, None) == -3
+    assert gt(one, one, one, one, one, 2, 4, -1, one, 4, None, one, 300, 500, 64, 0, 64, None) == -2
+    # the read-only yardstick validates like the launch it stands beside
+    arr = lambda v: (C.c_void_p * 1)(v)
+    pr = dzlib.dz_probe_read
+    n1 = (C.c_int * 1)(64)
+    assert pr(0, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 8, 512, 2, 2, 0, one, None) == -1
+    assert pr(1, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 8, 512, 2, 2, 0, None, None) == -1
+    assert pr(1, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 33, 512, 2, 2, 0, one, None) == -2
+    assert pr(1, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 8, 512, 2, 9, 0, one, None) == -2
+    assert pr(1, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 8, 512, 3, 2, 0, one, None) == -3
+    assert pr(1, arr(0x1000), arr(0x1000), arr(0x1000), arr(0x1000), n1, 8, 500, 2, 2, 0, one, None) == -2
+    assert pr(1, arr(0x1000), arr(None), arr(0x1000), arr(0x1000), n1, 8, 512, 2, 2, 0, one, None) == -1
 
 
 def test_compressor_entry_points_check_their_arguments(dzlib):

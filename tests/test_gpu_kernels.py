@@ -274,6 +274,25 @@ def test_prefill_sized_call(dev, kind):
     assert o.rel_err(y, ref) <= TOL
 
 
+@pytest.mark.parametrize("bits,with_x", [(2, 0), (2, 1), (4, 1)])
+def test_read_only_yardstick_runs_on_the_fused_launch_geometry(dev, bits, with_x):
+    """dz_probe_read: the launch bench.py times beside the fused kernel reads the tiled base weight and
+    the packed words of the first D slots with the fused kernel's grid and writes nothing (its sink
+    stays as it was)."""
+    import ctypes as C
+    from deltazip_amd import _lib
+    p1 = make_problem(256, 1024, bits, -1, 4, 32, "uniform", 3, dev)
+    p2 = make_problem(96, 1024, bits, -1, 4, 32, "uniform", 4, dev)
+    tiles = [ops.tile_base(p["wb"]) for p in (p1, p2)]
+    sink = torch.full((64,), 7, dtype=torch.int32, device=dev)
+    arr = lambda ts: (C.c_void_p * 2)(*[t.data_ptr() for t in ts])
+    rc = _lib.lib().dz_probe_read(2, arr([p1["x"], p2["x"]]), arr(tiles), arr([p1["q"], p2["q"]]),
+                                  arr([p1["m"], p2["m"]]), (C.c_int * 2)(256, 96), 32, 1024, bits, 4, with_x,
+                                  sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0 and bool((sink == 7).all())
+
+
 def test_row_blocks_made_once_per_batch(dev):
     """ops.row_blocks(indices, S) made once and passed as `order` to several calls gives, bit for
     bit, what each call gives when it orders the batch itself; blocks of another batch are refused."""
