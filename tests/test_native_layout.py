@@ -137,3 +137,30 @@ def test_gptq_writer_argument_checks(dzlib):
     with pytest.raises(ValueError):
         ops.unrepack_native_to_gptq(torch.zeros(10, dtype=torch.int32), torch.zeros(10, dtype=torch.int16),
                                     torch.zeros((1, 32), dtype=torch.float16), 256, 32, 4)
+
+
+def test_untile_base_inverts_the_documented_tile_order():
+    """ops.untile_base (plain tensor ops, runs anywhere) against the tile formula written out value by
+    value: tile (np, kb) of 16 KiB, fragment (s, j, h) of 1 KiB, lane 16*g + i holding
+    W[32*np + 16*s + i][256*kb + 64*j + 16*g + 8*h + e], e = 0..7."""
+    import torch
+    from deltazip_amd import ops
+    n, k = 64, 512
+    w = (np.arange(n * k, dtype=np.int64) % 30011).astype(np.float16).reshape(n, k)   # exact in fp16, no repeats per row block
+    tiled = np.empty(n * k, dtype=np.float16)
+    for np_ in range(n // 32):
+        for kb in range(k // 256):
+            for s in range(2):
+                for j in range(4):
+                    for h in range(2):
+                        for lane in range(64):
+                            i, g = lane % 16, lane // 16
+                            off = ((np_ * (k // 256) + kb) * 16384 + ((s * 4 + j) * 2 + h) * 1024 + lane * 16) // 2
+                            row, col = 32 * np_ + 16 * s + i, 256 * kb + 64 * j + 16 * g + 8 * h
+                            tiled[off:off + 8] = w[row, col:col + 8]
+    back = ops.untile_base(torch.from_numpy(tiled.reshape(n, k)))
+    assert np.array_equal(back.numpy(), w)
+    with pytest.raises(ValueError):
+        ops.untile_base(torch.zeros(48, 512, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        ops.untile_base(torch.zeros(64, 512, dtype=torch.float32))
