@@ -427,3 +427,36 @@ def test_manager_makes_row_blocks_once_for_a_large_batch(dev):
     assert mgr.row_blocks[0] is blocks          # made once, not per layer call
     mgr.set_delta_mapping(DeltaMapping(ids[:9], ids[:2]))
     assert mgr.row_blocks[0] is None
+
+
+@pytest.mark.gpu
+def test_manager_with_one_copy_of_the_base_weights(dev):
+    """DeltaConfig.keep_row_major_base=False through the manager: every wrapped projection frees its
+    row-major weight, and a decode-sized and a prefill-sized batch give, bit for bit, what a manager
+    that keeps both copies gives on the same weights and deltas."""
+    bits = 4
+    torch.manual_seed(7)
+    models = [ToyModel(dev), ToyModel(dev)]
+    models[1].load_state_dict(models[0].state_dict())
+    cfgs = [DeltaConfig(max_deltas=2, max_bitwidth=bits), DeltaConfig(max_deltas=2, max_bitwidth=bits,
+                                                                       keep_row_major_base=False)]
+    mgrs = [create_delta_manager(m, 8, 1024, V, c) for m, c in zip(models, cfgs)]
+    for mgr in mgrs:
+        for did in (11, 12):
+            mgr.add_delta(make_delta_model(did, bits, 100 * did)[0])
+            mgr.activate_delta(did)
+    qkv = [m.get_submodule("model.layers.0.self_attn.qkv_proj") for m in models]
+    assert qkv[0].base_layer.weight.numel() > 0 and qkv[1].base_layer.weight.numel() == 0
+    assert qkv[1].base_shape == tuple(qkv[0].base_layer.weight.shape)
+    rng = np.random.default_rng(11)
+    for T in (9, 700):
+        ids = tuple(int(i) for i in rng.choice([0, 11, 12], size=T))
+        x = torch.from_numpy(o.make_x(T, H, 5)).to(dev)
+        outs = []
+        for mgr, model in zip(mgrs, models):
+            mgr.set_delta_mapping(DeltaMapping(ids, ids[:2]))
+            outs.append([model.get_submodule("model.layers.0." + name)(x)[0]
+                         for name in ("self_attn.qkv_proj", "self_attn.o_proj", "mlp.gate_up_proj")])
+        torch.cuda.synchronize()
+        for a, b in zip(*outs):
+            assert torch.equal(a, b), T
